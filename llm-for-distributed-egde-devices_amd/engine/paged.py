@@ -1,0 +1,104 @@
+"""Paged cache and per-slot recurrent state for models that run ragged steps.
+
+One pool of ``num_pages`` pages of ``page`` tokens serves every live sequence: a sequence owns
+the pages its page-table row lists, takes a new one when its length crosses a page border and
+gives all of them back when it ends, so the pool is sized for the tokens alive at one time, not
+for (slots x longest sequence) as the row cache of ``engine.kv_cache`` is.  A page id addresses
+the same page in every run's tensors (a *run* is one execution of a layer: a looped layer has
+one run per pass, each with its own cache).
+
+Per run:
+  k [pages, page, kv heads, D], v [pages, page, kv heads, Dv]   activation dtype
+  k_pool / v_pool [pages, ceil(page / pool), kv heads, D | Dv]  fp32 block means; block b sits
+      beside the page of its first token b*pool, at entry (b*pool mod page) // pool
+  conv [slots, taps - 1, channels]                              the convolution's last inputs
+  ssm  [slots, heads, N, vdim] fp32                             the state-space matrix
+A slot's recurrent rows are not cleared on release: a portion that starts at position 0 ignores
+what the slot held (the kernels start from zero there).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+
+class RunCache:
+    __slots__ = ("k", "v", "k_pool", "v_pool", "conv", "ssm")
+
+
+class PagedCache:
+    def __init__(self, run_specs, num_pages: int, slots: int = 4, page: int = 64, dtype=torch.bfloat16,
+                 device=None):
+        self.page, self.num_pages, self.slots = page, num_pages, slots
+        self.dtype, self.device = dtype, device
+        self.runs: List[RunCache] = []
+        for s in run_specs:
+            rc = RunCache()
+            a, m = s.attn, s.ssd
+            rc.k = torch.zeros(num_pages, page, a.kv_heads, a.dim, dtype=dtype, device=device)
+            rc.v = torch.zeros(num_pages, page, a.kv_heads, a.vdim, dtype=dtype, device=device)
+            if a.window is not None and a.pool:
+                pb = (page + a.pool - 1) // a.pool
+                rc.k_pool = torch.zeros(num_pages, pb, a.kv_heads, a.dim, dtype=torch.float32, device=device)
+                rc.v_pool = torch.zeros(num_pages, pb, a.kv_heads, a.vdim, dtype=torch.float32, device=device)
+            else:
+                rc.k_pool = rc.v_pool = None
+            rc.conv = torch.zeros(slots, max(m.conv - 1, 1), m.conv_channels, dtype=dtype, device=device)
+            rc.ssm = torch.zeros(slots, m.heads, m.state, m.vdim, dtype=torch.float32, device=device)
+            self.runs.append(rc)
+        # a sequence may grow until it holds every page
+        self.page_table = torch.zeros(slots, num_pages, dtype=torch.int32, device=device)
+        self._table_host = [[] for _ in range(slots)]           # pages of each slot, in order
+        self.free_pages = list(range(num_pages - 1, -1, -1))     # pop() hands out low ids first
+        self.free_slots = list(range(slots - 1, -1, -1))
+        self.lens = [0] * slots
+
+    def run(self, r: int) -> RunCache:
+        return self.runs[r]
+
+    # ------------------------------------------------------------------ slots and pages
+    def acquire(self) -> int:
+        if not self.free_slots:
+            raise RuntimeError("no free state slot")
+        s = self.free_slots.pop()
+        self.lens[s] = 0
+        return s
+
+    def pages_for(self, n: int) -> int:
+        return (n + self.page - 1) // self.page
+
+    def can_extend(self, slot: Optional[int], new_len: int) -> bool:
+        have = len(self._table_host[slot]) if slot is not None else 0
+        return self.pages_for(new_len) - have <= len(self.free_pages)
+
+    def extend(self, slot: int, new_len: int) -> None:
+        """Make room for positions [0, new_len) of the slot's sequence."""
+        own = self._table_host[slot]
+        need = self.pages_for(new_len) - len(own)
+        if need > len(self.free_pages):
+            raise RuntimeError(f"page pool exhausted: {need} pages wanted, {len(self.free_pages)} free")
+        if need > 0:
+            first = len(own)
+            own.extend(self.free_pages.pop() for _ in range(need))
+            self.page_table[slot, first:len(own)] = torch.tensor(own[first:], dtype=torch.int32)
+        self.lens[slot] = max(self.lens[slot], new_len)
+
+    def release(self, slot: int) -> None:
+        self.free_pages.extend(reversed(self._table_host[slot]))
+        self._table_host[slot] = []
+        self.lens[slot] = 0
+        self.free_slots.append(slot)
+
+    def nbytes(self) -> int:
+        n = self.page_table.numel() * 4
+        for rc in self.runs:
+            for name in RunCache.__slots__:
+                t = getattr(rc, name)
+                if t is not None:
+                    n += t.numel() * t.element_size()
+        return n
+
+    def stats(self) -> Dict[str, int]:
+        return {"pages": self.num_pages, "free_pages": len(self.free_pages), "slots": self.slots,
+                "free_slots": len(self.free_slots)}

@@ -18,7 +18,77 @@ import dataclasses
 import json
 import os
 from dataclasses import dataclass, field
-from typing import Optional
+from typing import List, Optional
+
+
+@dataclass
+class WindowAttnSpec:
+    """Softmax attention over a sliding window plus one pooled key / value per block of ``pool``
+    tokens that lies wholly before the window (``window`` None: plain causal attention; ``pool``
+    None: nothing beyond the window), grouped-query heads, a per-head sigmoid output gate and
+    rotary positions on the first ``rot_dims`` coordinates (``rot_scaling``: YaRN constants)."""
+    heads: int
+    kv_heads: int
+    dim: int                     # query / key size per head
+    vdim: int                    # value size per head
+    scale: float
+    window: Optional[int] = None
+    pool: Optional[int] = None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[dict] = None   # {"rope_type": "yarn", factor, original, fast, slow}
+    gate: bool = True
+
+    @property
+    def proj_sizes(self):
+        """Row blocks of the fused input projection: q | k | v | gate."""
+        return (self.heads * self.dim, self.kv_heads * self.dim, self.kv_heads * self.vdim,
+                self.heads if self.gate else 0)
+
+
+@dataclass
+class SSDSpec:
+    """Mamba-2 (state-space duality) mixer: ``heads`` heads of ``vdim`` channels, state size
+    ``state`` per channel, B / C shared by ``heads / groups`` heads, a causal depthwise convolution
+    of ``conv`` taps over x | B | C, and an RMS norm in ``norm_groups`` parts after the gate."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    @property
+    def in_size(self) -> int:
+        """Rows of the input projection: z | x | B | C | dt."""
+        return 2 * self.inner + 2 * self.groups * self.state + self.heads
+
+
+@dataclass
+class LayerSpec:
+    """One layer of a ``layer_specs`` model: the mixer kind with its branches, and the feed-forward
+    width (None: the layer has no feed-forward)."""
+    mixer: str                               # "parallel": attention and state-space side by side
+    attn: Optional[WindowAttnSpec] = None
+    ssd: Optional[SSDSpec] = None
+    ff: Optional[int] = None
+    ff_act: str = "relu2"
+
+
+@dataclass
+class LoopSpec:
+    """Layers [start, stop) run ``times`` times in a row with the same weights."""
+    start: int
+    stop: int
+    times: int
 
 
 @dataclass
@@ -49,6 +119,22 @@ class ModelConfig:
     bos_token_id: Optional[int] = None
     eos_token_id: Optional[int] = None
     name: str = ""
+    # per-layer descriptions (arch "nudadra"): every layer has its own mixer geometry, the stack may
+    # repeat a span of layers, the embedding is scaled and the norms carry one gain
+    layer_specs: Optional[List[LayerSpec]] = None
+    loop: Optional[LoopSpec] = None
+    embed_scale: float = 1.0
+
+    def layer_runs(self) -> List[tuple]:
+        """[(layer index, pass number or None)] in execution order; every run has its own cache."""
+        n = self.num_layers
+        if self.loop is None:
+            return [(i, None) for i in range(n)]
+        lp = self.loop
+        runs = [(i, None) for i in range(lp.start)]
+        for t in range(lp.times):
+            runs += [(i, t) for i in range(lp.start, lp.stop)]
+        return runs + [(i, None) for i in range(lp.stop, n)]
 
     def __post_init__(self):
         if self.head_dim is None:
@@ -224,8 +310,70 @@ def _rope_params(c: dict, default_theta: float, default_partial: float = 1.0):
     return float(theta), float(partial), scaling
 
 
+def from_nudadra_config(c: dict) -> ModelConfig:
+    """The Nudadra layout of ``config.json``: ``layers`` (one entry per layer: ``type``, ``mixer``
+    with ``left`` = attention and ``right`` = state-space sizes, ``mlp`` or null), ``loop``,
+    ``embedding.scale``, ``norm.eps``, ``vocab``, ``width``."""
+    specs = []
+    for l in c["layers"]:
+        if l["type"] != "parallel":
+            raise ValueError(f"unsupported layer type {l['type']!r}")
+        a, r = l["mixer"]["left"], l["mixer"]["right"]
+        rot, mask = a.get("rot") or None, a.get("mask") or {}
+        sc = (rot or {}).get("scaling") or None
+        attn = WindowAttnSpec(heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]),
+                              vdim=int(a["vdim"]), scale=float(a["scale"]),
+                              window=int(mask["size"]) if mask.get("size") is not None else None,
+                              pool=int(mask["pool"]) if mask.get("pool") else None,
+                              rot_dims=int(rot["dims"]) if rot else 0,
+                              rot_base=float(rot["base"]) if rot else 10000.0,
+                              rot_scaling=dict(sc, rope_type="yarn") if sc else None)
+        ssd = SSDSpec(heads=int(r["heads"]), vdim=int(r["vdim"]), state=int(r["state"]), groups=int(r["groups"]),
+                      conv=int(r["conv"]), norm_groups=int(r["norm_groups"]))
+        mlp = l.get("mlp") or None
+        if mlp and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}")
+        specs.append(LayerSpec("parallel", attn, ssd, int(mlp["ff"]) if mlp else None))
+    lp = c.get("loop") or None
+    a0 = specs[0].attn
+    return ModelConfig(arch="nudadra", vocab_size=int(c["vocab"]), hidden_size=int(c["width"]),
+                       num_layers=len(specs), num_heads=a0.heads, num_kv_heads=a0.kv_heads,
+                       intermediate_size=specs[0].ff or 0, head_dim=a0.dim, max_position_embeddings=1 << 20,
+                       norm="rms_scalar", norm_eps=float(c["norm"]["eps"]), act="relu2", parallel_residual=True,
+                       shared_input_norm=True, rotary_dim=a0.rot_dims, rope_theta=a0.rot_base,
+                       name=c.get("name", "nudadra"), layer_specs=specs,
+                       loop=LoopSpec(int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else None,
+                       embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)))
+
+
+def to_nudadra_config(cfg: ModelConfig) -> dict:
+    """Inverse of ``from_nudadra_config``."""
+    layers = []
+    for s in cfg.layer_specs:
+        a, r = s.attn, s.ssd
+        left = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale}
+        if a.window is not None:
+            left["mask"] = {"size": a.window, "pool": a.pool}
+        if a.rot_dims:
+            left["rot"] = {"dims": a.rot_dims, "base": a.rot_base}
+            if a.rot_scaling:
+                left["rot"]["scaling"] = {k: v for k, v in a.rot_scaling.items() if k != "rope_type"}
+        right = {"heads": r.heads, "vdim": r.vdim, "state": r.state, "groups": r.groups, "conv": r.conv,
+                 "norm_groups": r.norm_groups}
+        layers.append({"type": "parallel", "mixer": {"left": left, "right": right},
+                       "mlp": {"kind": "dense", "ff": s.ff} if s.ff else None})
+    out = {"architecture": "Nudadra", "vocab": cfg.vocab_size, "width": cfg.hidden_size, "layers": layers,
+           "norm": {"eps": cfg.norm_eps}, "embedding": {"scale": cfg.embed_scale}}
+    if cfg.loop is not None:
+        out["loop"] = {"start": cfg.loop.start, "stop": cfg.loop.stop, "times": cfg.loop.times}
+    return out
+
+
 def from_hf_config(c: dict) -> ModelConfig:
-    """Map a Hugging Face ``config.json`` onto ModelConfig."""
+    """Map a ``config.json`` onto ModelConfig (Hugging Face ``model_type`` layouts, or an
+    ``architecture`` key naming a per-layer layout)."""
+    if str(c.get("architecture", "")).lower() == "nudadra":
+        return from_nudadra_config(c)
     mt = c.get("model_type")
     eos = c.get("eos_token_id")
     if isinstance(eos, list):

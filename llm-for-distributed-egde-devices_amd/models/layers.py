@@ -256,6 +256,19 @@ class Norm(nn.Module):
         return ops.layer_norm(x, self.weight, self.bias, self.eps, residual)
 
 
+class ScalarNorm(nn.Module):
+    """RMS norm whose gain is one number for all coordinates: fp32 rows in (the residual stream of
+    the layer-spec models), rows of the consumer's dtype out."""
+
+    def __init__(self, eps: float, device=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(1, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, x: torch.Tensor, out_dtype=torch.bfloat16) -> torch.Tensor:
+        return ops.seqmix.scalar_rms_norm(x, self.weight, self.eps, out_dtype)
+
+
 def act_fn(x, act: str, quant: bool):
     if quant:
         q, s = ops.activation_quant(x, act)

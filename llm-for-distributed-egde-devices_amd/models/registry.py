@@ -39,12 +39,13 @@ def preset_for(name: str) -> Optional[str]:
     return None
 
 
-def precision_dtype(precision: str, device, quant: str = "none") -> torch.dtype:
+def precision_dtype(precision: str, device, quant: str = "none", fp32_ok: bool = False) -> torch.dtype:
     """torch dtype of a model's 16-bit tensors for the reference's ``precision`` flag
     (combine_model_fp_updated.py:32-34: fp16 unless "bf16"; phi2-pythia_fp_updated.py:32).  The
     GPU runs fp16 and bf16 models on their own kernel instantiations (fp16 MFMA GEMV / attention,
     fp16 norms and RoPE).  Quantised models (``quant`` != none) keep bf16 activations on the GPU:
-    the INT8 GEMM epilogues write bf16."""
+    the INT8 GEMM epilogues write bf16.  ``fp32_ok``: the model's kernels have fp32 instantiations
+    (the ragged-step kernels of the layer-spec models do)."""
     p = (precision or "bf16").lower()
     dev = torch.device(device) if device is not None else torch.device("cpu")
     want = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}.get(p, torch.bfloat16)
@@ -52,7 +53,7 @@ def precision_dtype(precision: str, device, quant: str = "none") -> torch.dtype:
         if quant not in (None, "none") and want != torch.bfloat16:
             log.info(f"precision {p} with --quant {quant}: the INT8 kernels run bf16 activations")
             return torch.bfloat16
-        if want == torch.float32:
+        if want == torch.float32 and not fp32_ok:
             log.info("precision fp32 on the GPU: the HIP kernels run 16-bit; using bf16")
             return torch.bfloat16
     return want
@@ -87,8 +88,14 @@ def load_model(name_or_path: str, precision: str = "bf16", quant: str = "none", 
         if quant not in (None, "none", model.quant_mode):
             log.warning(f"{qdir} holds {model.quant_mode} weights: --quant {quant} ignored")
         return model, load_tokenizer(qdir, model.cfg.vocab_size), f"int8-checkpoint:{qdir}"
-    dtype = precision_dtype(precision, device, quant)
     path = resolve_model_dir(name_or_path, base_dir)
+    spec_model = False
+    if path is not None:
+        from .configs import from_hf_dir
+        spec_model = from_hf_dir(path).layer_specs is not None
+    dtype = precision_dtype(precision, device, quant, fp32_ok=spec_model)
+    if spec_model and quant not in (None, "none"):
+        raise ValueError("layer-spec models run bf16 or fp32 (no INT8 path)")
     if path is not None:
         assert units is None, "half-layer stages of HF checkpoints: load the whole layers"
         model = load_hf_model(path, dtype=dtype, device=device, first=first, last=last)

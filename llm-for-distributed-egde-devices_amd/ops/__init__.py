@@ -704,3 +704,5 @@ def embedding(ids, table, out_f32: bool = False):
 
 
 rope_tables = _ref.rope_tables
+
+from . import seqmix  # noqa: E402  (ragged-step ops of the layer-spec models)

@@ -134,8 +134,20 @@ def gelu_quant(x: torch.Tensor, approximate: str = "tanh"):
 def rope_tables(rotary_dim: int, max_pos: int, theta: float, scaling: Optional[dict] = None,
                 device=None) -> torch.Tensor:
     """cos/sin table [max_pos, rotary_dim/2, 2] f32, HF "rotate_half" convention,
-    with Llama-3 frequency scaling when ``scaling['rope_type'] == 'llama3'``."""
+    with Llama-3 frequency scaling when ``scaling['rope_type'] == 'llama3'`` and the YaRN blend
+    (``'yarn'``: factor, original, fast, slow; cos and sin carry the 0.1 ln(factor) + 1 gain)."""
     inv = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2, dtype=torch.float64) / rotary_dim))
+    gain = 1.0
+    if scaling and scaling.get("rope_type", scaling.get("type")) == "yarn":
+        # pair i keeps its frequency below the pair that makes `fast` turns over the original
+        # context and is divided by `factor` above the pair that makes `slow` turns; linear between
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        pair_of = lambda turns: rotary_dim * math.log(orig / (2 * math.pi * turns)) / (2 * math.log(theta))
+        lo = max(math.floor(pair_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(scaling["slow"]))), rotary_dim - 1)
+        ramp = ((torch.arange(rotary_dim // 2, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        inv = inv / factor * ramp + inv * (1 - ramp)
+        gain = 0.1 * math.log(factor) + 1.0
     if scaling and scaling.get("rope_type", scaling.get("type")) == "llama3":
         factor = scaling["factor"]
         lo, hi = scaling["low_freq_factor"], scaling["high_freq_factor"]
@@ -151,7 +163,7 @@ def rope_tables(rotary_dim: int, max_pos: int, theta: float, scaling: Optional[d
         inv = inv / scaling["factor"]
     t = torch.arange(max_pos, dtype=torch.float64)
     ang = torch.outer(t, inv)
-    return torch.stack([ang.cos(), ang.sin()], -1).float().to(device)
+    return (torch.stack([ang.cos(), ang.sin()], -1) * gain).float().to(device)
 
 
 def _rotate(x: torch.Tensor, cs: torch.Tensor, rotary_dim: int) -> torch.Tensor:

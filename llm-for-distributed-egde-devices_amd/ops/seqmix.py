@@ -1,0 +1,309 @@
+"""Ops of the sequence-mixing layers that run over a ragged step and a paged cache.
+
+A step is a flat run of tokens from several sequences (``RaggedMeta``): each sequence brings a
+portion of new tokens (a whole prompt, a cut of one, or a single decoded token) that continues
+what the cache and the recurrent state hold for its slot.  Keys and values live in pages of
+``page`` tokens shared by all sequences through a page table; a pooled key / value per block of
+tokens sits beside the page that holds the block's first token; recurrent state (convolution
+tail, state-space matrix) lives in per-slot rows.
+
+GPU tensors run the kernels in ``csrc/seqmix*.hip`` (fp32 or bf16 storage, fp32 math for
+scores, norms, decays and state); CPU tensors run the PyTorch forms below, which define the
+semantics the kernels are tested against.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+
+def _ops():
+    from .. import ops
+    return ops
+
+
+def _gpu(t: torch.Tensor) -> bool:
+    return _ops().gpu_path(t)
+
+
+def _ext():
+    return _ops().ext()
+
+
+@dataclass
+class RaggedMeta:
+    """One step's layout.  Sequence i of the step sits in state slot ``seq_slot[i]``, brings
+    ``seq_len[i]`` tokens at flat rows ``seq_off[i]..`` for positions ``seq_start[i]..``."""
+    n: int
+    T: int
+    seq_slot: torch.Tensor        # int32 [n]
+    seq_start: torch.Tensor       # int32 [n]
+    seq_len: torch.Tensor         # int32 [n]
+    seq_off: torch.Tensor         # int32 [n]
+    tok_seq: torch.Tensor         # int32 [T] index into the step's sequences
+    tok_pos: torch.Tensor         # int32 [T] position in its sequence
+    page_table: torch.Tensor      # int32 [slots, pages per sequence]
+    page: int
+    host: List[Tuple[int, int, int, int]]   # (slot, start, len, off) per sequence
+    max_len: int                  # longest portion of the step
+    max_keys: int                 # most keys any sequence holds after the step
+
+    @classmethod
+    def build(cls, seqs: List[Tuple[int, int, int]], page_table: torch.Tensor, page: int, device) -> "RaggedMeta":
+        """``seqs``: (slot, start, len) per sequence, in flat-row order.  One host -> device copy."""
+        host, off = [], 0
+        for slot, start, n in seqs:
+            host.append((slot, start, n, off))
+            off += n
+        T, n = off, len(seqs)
+        flat = [h[0] for h in host] + [h[1] for h in host] + [h[2] for h in host] + [h[3] for h in host]
+        for i, (_, start, ln, _) in enumerate(host):
+            flat += [i] * ln
+        for (_, start, ln, _) in host:
+            flat += list(range(start, start + ln))
+        buf = torch.tensor(flat, dtype=torch.int32)
+        if torch.device(device).type == "cuda":
+            buf = buf.pin_memory().to(device, non_blocking=True)
+        s = lambda a, b: buf[a:b]
+        return cls(n, T, s(0, n), s(n, 2 * n), s(2 * n, 3 * n), s(3 * n, 4 * n), s(4 * n, 4 * n + T),
+                   s(4 * n + T, 4 * n + 2 * T), page_table, page, host, max(h[2] for h in host),
+                   max(h[1] + h[2] for h in host))
+
+
+# --------------------------------------------------------------------------- element-wise pieces
+def embedding_scaled(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    """fp32 rows ``table[ids] * scale`` (the residual stream starts in 32-bit)."""
+    if _gpu(table):
+        return _ext().sm_embed(ids.long().contiguous(), table, float(scale))
+    return table[ids.long()].float() * scale
+
+
+def scalar_rms_norm(x: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """x fp32 [T, W] / sqrt(mean(x^2) + eps) * gain (one number), stored as ``out_dtype``."""
+    if _gpu(x):
+        return _ext().sm_scalar_norm(x, gain.reshape(1), float(eps), out_dtype == torch.float32)
+    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * gain.float().reshape(())
+    return y.to(out_dtype)
+
+
+def relu2(u: torch.Tensor, c0: int = 0, C: Optional[int] = None) -> torch.Tensor:
+    """max(x, 0)^2 of columns [c0, c0 + C) of u [T, *] (squared in fp32, stored contiguous in u's dtype)."""
+    C = u.shape[1] - c0 if C is None else C
+    if _gpu(u):
+        return _ext().sm_relu2(u, int(c0), int(C))
+    return torch.relu(u[:, c0:c0 + C].float()).pow(2).to(u.dtype)
+
+
+def linear_f32(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T, K] @ weight[N, K]^T (+ bias fp32 [N]) with an fp32 result: the products accumulate in
+    fp32 and the sum is not rounded to the inputs' 16-bit type (a projection that writes the
+    residual stream)."""
+    if x.dtype == torch.float32:
+        y = F.linear(x, weight)
+    elif x.is_cuda:
+        global _MM_F32
+        if _MM_F32 is None:
+            try:
+                torch.mm(x[:1], weight[:1].t(), out_dtype=torch.float32)
+                _MM_F32 = True
+            except (RuntimeError, TypeError):
+                _MM_F32 = False
+        y = torch.mm(x, weight.t(), out_dtype=torch.float32) if _MM_F32 else F.linear(x, weight).float()
+    else:
+        y = F.linear(x.float(), weight.float())
+    return y if bias is None else y.add_(bias)
+
+
+_MM_F32: Optional[bool] = None
+
+
+def cat_cast(a: torch.Tensor, b: torch.Tensor, dtype) -> torch.Tensor:
+    """[a | b] of two fp32 [T, W] streams as ``dtype`` [T, 2 W] (a projection's input)."""
+    if _gpu(a):
+        return _ext().sm_cat_cast(a, b, dtype == torch.float32)
+    return torch.cat([a, b], -1).to(dtype)
+
+
+def combine_residual(x: torch.Tensor, left: torch.Tensor, right: torch.Tensor, wl: torch.Tensor,
+                     wr: torch.Tensor, eps: float, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x (fp32 [T, W], updated in place) += 0.5 (rms(left) wl + rms(right) wr) + extra: the two
+    branch outputs are each divided by their own root mean square over the width."""
+    if _gpu(x):
+        _ext().sm_combine(x, left, right, wl, wr, float(eps), extra)
+        return x
+    l, r = left.float(), right.float()
+    l = l * torch.rsqrt(l.pow(2).mean(-1, keepdim=True) + eps) * wl.float()
+    r = r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps) * wr.float()
+    y = 0.5 * (l + r)
+    if extra is not None:
+        y = y + extra.float()
+    x.add_(y)
+    return x
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, groups: int, eps: float,
+                     out_dtype) -> torch.Tensor:
+    """rms-norm in ``groups`` equal parts of (y * silu(z)) times weight.  y fp32 [T, C]; z [T, C] a
+    (possibly strided) view in the activation dtype."""
+    if _gpu(y):
+        return _ext().sm_gated_norm(y, z, weight, int(groups), float(eps), out_dtype == torch.float32)
+    T, C = y.shape
+    g = (y * F.silu(z.float())).view(T, groups, C // groups)
+    g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+    return (g.view(T, C) * weight.float()).to(out_dtype)
+
+
+# --------------------------------------------------------------------------- attention side
+def _rotate_half(x, cs, dims):
+    half = dims // 2
+    u, v = x[..., :half], x[..., half:dims]
+    c, s = cs[..., 0], cs[..., 1]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
+
+
+def rope_paged_write(proj: torch.Tensor, meta: RaggedMeta, rope: Optional[torch.Tensor], k_pages: torch.Tensor,
+                     v_pages: torch.Tensor, heads: int, rot_dims: int) -> torch.Tensor:
+    """proj [T, q | k | v | ...] -> rotated q [T, heads, D]; the rotated keys and the values go
+    to their pages ``[pages, page, kv heads, D | Dv]`` at each token's position."""
+    G, D, Dv = k_pages.shape[2], k_pages.shape[3], v_pages.shape[3]
+    if _gpu(proj):
+        return _ext().sm_rope_write(proj, meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.page_table,
+                                    rope if rot_dims else None, k_pages, v_pages, int(heads), int(rot_dims))
+    T = proj.shape[0]
+    x = proj.float()
+    q = x[:, :heads * D].view(T, heads, D)
+    k = x[:, heads * D:(heads + G) * D].view(T, G, D)
+    v = x[:, (heads + G) * D:(heads + G) * D + G * Dv].view(T, G, Dv)
+    pos = meta.tok_pos.long()
+    if rope is not None and rot_dims:
+        cs = rope[pos][:, None]
+        q, k = _rotate_half(q, cs, rot_dims), _rotate_half(k, cs, rot_dims)
+    slot = meta.seq_slot.long()[meta.tok_seq.long()]
+    pid = meta.page_table[slot, pos // meta.page].long()
+    k_pages[pid, pos % meta.page] = k.to(k_pages.dtype)
+    v_pages[pid, pos % meta.page] = v.to(v_pages.dtype)
+    return q.to(proj.dtype)
+
+
+def pool_blocks(k_pages, v_pages, k_pool, v_pool, meta: RaggedMeta, pool: int) -> None:
+    """Mean key and value (fp32) of every block of ``pool`` tokens whose last token this step wrote,
+    taken over the rows as the pages hold them; block b lands beside the page of its first token,
+    at entry (b pool mod page) // pool."""
+    if _gpu(k_pages):
+        _ext().sm_pool_blocks(k_pages, v_pages, k_pool, v_pool, meta.seq_slot, meta.seq_start, meta.seq_len,
+                              meta.page_table, int(pool), int(meta.n), int((meta.max_len + pool - 1) // pool + 1))
+        return
+    page = meta.page
+    for slot, start, n, _ in meta.host:
+        b = start // pool                                # first block whose last token >= start
+        while b * pool + pool - 1 < start + n:
+            pos = torch.arange(b * pool, (b + 1) * pool, device=k_pages.device)
+            pid = meta.page_table[slot, pos // page].long()
+            first = meta.page_table[slot, (b * pool) // page].long()
+            e = ((b * pool) % page) // pool
+            k_pool[first, e] = k_pages[pid, pos % page].float().mean(0)
+            v_pool[first, e] = v_pages[pid, pos % page].float().mean(0)
+            b += 1
+
+
+def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages, v_pages, k_pool, v_pool,
+                          meta: RaggedMeta, scale: float, window: Optional[int], pool: Optional[int]) -> torch.Tensor:
+    """q [T, H, D] -> [T, H * Dv].  Query position i sees the tokens j with 0 <= i - j < window and
+    the pooled blocks b with b pool + pool - 1 <= i - window, in one softmax (fp32); head h's result
+    is multiplied by sigmoid(gate[t, h]) when ``gate`` ([T, H] view) is given."""
+    T, H, D = q.shape
+    G, Dv = k_pages.shape[2], v_pages.shape[3]
+    if _gpu(q):
+        return _ext().sm_attention(q, gate, k_pages, v_pages, k_pool if pool else None, v_pool if pool else None,
+                                   meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.page_table, float(scale),
+                                   int(window) if window is not None else 0, int(pool or 0), int(meta.max_keys))
+    page = meta.page
+    out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
+    R = H // G
+    for slot, start, n, off in meta.host:
+        L = start + n
+        pos = torch.arange(L, device=q.device)
+        pid = meta.page_table[slot, pos // page].long()
+        k = k_pages[pid, pos % page].float()                     # [L, G, D]
+        v = v_pages[pid, pos % page].float()
+        qi = q[off:off + n].float().view(n, G, R, D)
+        i = torch.arange(start, L, device=q.device)
+        s = torch.einsum("ngrd,lgd->ngrl", qi, k) * scale
+        d = i[:, None] - pos[None]
+        vis = d >= 0
+        if window is not None:
+            vis &= d < window
+        s = s.masked_fill(~vis[:, None, None, :], float("-inf"))
+        vals = v
+        if window is not None and pool:
+            nb = max((L - 1 - window + 1) // pool, 0)
+            if nb > 0:
+                bp = torch.arange(nb, device=q.device) * pool
+                first = meta.page_table[slot, bp // page].long()
+                kb = k_pool[first, (bp % page) // pool]           # [nb, G, D] fp32
+                vb = v_pool[first, (bp % page) // pool]
+                sb = torch.einsum("ngrd,bgd->ngrb", qi, kb) * scale
+                seen = (bp[None] + pool - 1) <= (i[:, None] - window)
+                sb = sb.masked_fill(~seen[:, None, None, :], float("-inf"))
+                s = torch.cat([s, sb], -1)
+                vals = torch.cat([v, vb], 0)
+        p = torch.softmax(s, -1)
+        out[off:off + n] = torch.einsum("ngrl,lgd->ngrd", p, vals).reshape(n, H, Dv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[..., None]
+    return out.reshape(T, H * Dv).to(q.dtype)
+
+
+# --------------------------------------------------------------------------- state-space side
+def conv_silu(u: torch.Tensor, c0: int, C: int, weight: torch.Tensor, bias: torch.Tensor, state: torch.Tensor,
+              meta: RaggedMeta) -> torch.Tensor:
+    """Causal depthwise convolution + silu over columns [c0, c0 + C) of u [T, *].  weight [C, taps]
+    (last tap = the current token), state [slots, taps - 1, C] = each slot's last inputs (zeros
+    before a sequence's start; a portion starting at 0 ignores what the slot held).  Returns
+    [T, C] and leaves the inputs of each sequence's last taps - 1 positions in ``state``."""
+    taps = weight.shape[1]
+    if _gpu(u):
+        out = _ext().sm_conv_silu(u, int(c0), int(C), weight, bias, state, meta.tok_seq, meta.tok_pos, meta.seq_slot,
+                                  meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n))
+        return out
+    out = torch.empty(u.shape[0], C, dtype=u.dtype, device=u.device)
+    w, b = weight.float(), bias.float()
+    for slot, start, n, off in meta.host:
+        x = u[off:off + n, c0:c0 + C].float()
+        hist = state[slot].float() if start > 0 else torch.zeros(taps - 1, C, device=u.device)
+        xin = torch.cat([hist, x], 0)                             # [taps - 1 + n, C]
+        win = xin.unfold(0, taps, 1)                              # [n, C, taps]
+        out[off:off + n] = F.silu((win * w[None]).sum(-1) + b).to(u.dtype)
+        state[slot] = xin[xin.shape[0] - (taps - 1):].to(state.dtype)
+    return out
+
+
+def ssd_scan(xbc: torch.Tensor, u: torch.Tensor, dt0: int, dt_bias, A_log, D, state: torch.Tensor,
+             meta: RaggedMeta, heads: int, vdim: int, N: int, groups: int) -> torch.Tensor:
+    """The state-space recurrence, token by token in fp32.  xbc [T, x | B | C] (after conv + silu),
+    the step sizes are columns [dt0, dt0 + heads) of u before softplus(. + dt_bias).  Per head:
+    S <- exp(-exp(A_log) dt) S + dt B x^T ; y = S^T C + D x.  state [slots, heads, N, vdim] fp32 is
+    read (zero for a portion starting at 0) and left at the portion's end.  Returns y fp32 [T, inner]."""
+    inner = heads * vdim
+    if _gpu(xbc):
+        return _ext().sm_ssd_scan(xbc, u, int(dt0), dt_bias, A_log, D, state, meta.seq_slot, meta.seq_start,
+                                  meta.seq_len, meta.seq_off, int(meta.n), int(heads), int(vdim), int(N), int(groups))
+    T = xbc.shape[0]
+    y = torch.empty(T, inner, dtype=torch.float32, device=xbc.device)
+    a = torch.exp(A_log.float())
+    rep = heads // groups
+    for slot, start, n, off in meta.host:
+        x = xbc[off:off + n, :inner].float().view(n, heads, vdim)
+        B = xbc[off:off + n, inner:inner + groups * N].float().view(n, groups, N).repeat_interleave(rep, 1)
+        C = xbc[off:off + n, inner + groups * N:].float().view(n, groups, N).repeat_interleave(rep, 1)
+        dt = F.softplus(u[off:off + n, dt0:dt0 + heads].float() + dt_bias.float(), threshold=1e9)
+        S = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+        for t in range(n):
+            decay = torch.exp(-a * dt[t])
+            S = decay[:, None, None] * S + (dt[t][:, None] * B[t])[:, :, None] * x[t][:, None, :]
+            y[off + t] = (torch.einsum("hnp,hn->hp", S, C[t]) + D.float()[:, None] * x[t]).reshape(inner)
+        state[slot] = S
+    return y
