@@ -36,8 +36,13 @@ def main(argv=None) -> int:
     ap.add_argument("--device", default=None, help="default: cuda:0 when a GPU is present")
     a = ap.parse_args(argv)
 
+    from .. import ops
     from ..engine.ragged import RaggedEngine
     from ..models.registry import load_model
+
+    # this program runs ragged-step models only: their kernels are a library of their own, built on
+    # first use; the projections take the vendor GEMM when the main kernel library was never built
+    ops.require_main_ext(False)
 
     dev = torch.device(a.device) if a.device else torch.device("cuda:0" if torch.cuda.is_available() else "cpu")
     torch.backends.cuda.matmul.allow_tf32 = False            # float32 means fp32 products

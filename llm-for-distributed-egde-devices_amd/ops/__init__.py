@@ -58,6 +58,15 @@ def available() -> bool:
 
 _REF_ON_GPU = os.environ.get("EDGELLM_REF_ON_GPU", "0") == "1"
 
+# False: 16-bit projections take the vendor GEMM when the main kernel library is absent instead of
+# raising (set by programs that run only layer-spec models, whose kernels are a library of their own)
+_MAIN_EXT_REQUIRED = True
+
+
+def require_main_ext(flag: bool) -> None:
+    global _MAIN_EXT_REQUIRED
+    _MAIN_EXT_REQUIRED = bool(flag)
+
 
 def _gpu(t: torch.Tensor) -> bool:
     return t.is_cuda and not _REF_ON_GPU
@@ -410,6 +419,8 @@ def bf16_decode_mode(x: torch.Tensor, weight: torch.Tensor, glu: bool = False, s
     if not (_gpu(x) and x.dtype in (torch.bfloat16, torch.float16) and weight.dtype == x.dtype
             and x.is_contiguous() and K % 64 == 0 and weight.shape[0] % (32 if glu else 16) == 0):
         return 0
+    if not available() and not _MAIN_EXT_REQUIRED:
+        return 0            # a process that built only the ragged-step library: vendor GEMM
     M = x.numel() // max(K, 1)
     if 0 < M <= BF16_GEMV_MAX_ROWS:
         return 1

@@ -6,6 +6,10 @@ host-only) is compiled once; everything is linked against torch's own HIP runtim
 ``ops/_C<EXT_SUFFIX>`` next to this file, so the built library travels with the repo snapshot.
 Cross-compiles without a GPU.
 
+Two libraries: ``_C`` (everything directly under ``csrc/``) and ``_seqmix`` (``csrc/seqmix/``: the
+ragged-step kernels of the layer-spec models, with their own bindings), so a process that runs
+only such a model compiles and loads only that one.
+
     python -m edgellm.ops.build            # or: python llm-for-distributed-egde-devices_amd/ops/build.py
 """
 from __future__ import annotations
@@ -35,8 +39,15 @@ def _torch_paths():
     return inc, lib, abi
 
 
-def target_path() -> str:
-    return os.path.join(HERE, "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+# hipcc -O3 forms packed fp32 instructions from plain float code; the ragged-step kernels are built
+# without them (their fp32 results are compared at 1e-5)
+SEQMIX_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+TARGETS = {"main": ("_C", CSRC, []), "seqmix": ("_seqmix", os.path.join(CSRC, "seqmix"), SEQMIX_FLAGS)}
+
+
+def target_path(target: str = "main") -> str:
+    return os.path.join(HERE, TARGETS[target][0] + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
 def _stale(obj: str, deps) -> bool:
@@ -53,22 +64,32 @@ def _run(cmd):
     return r.stdout
 
 
-def build(verbose: bool = False, jobs: int = 8) -> str:
-    os.makedirs(BUILD, exist_ok=True)
+def build(verbose: bool = False, jobs: int = 8, targets=("main", "seqmix")) -> str:
+    """Compile and link ``targets``; returns the path of the last one built."""
+    out = ""
+    for t in targets:
+        out = _build_target(t, verbose, jobs)
+    return out
+
+
+def _build_target(target: str, verbose: bool, jobs: int) -> str:
+    name, src_dir, extra = TARGETS[target]
+    build_dir = BUILD if target == "main" else os.path.join(BUILD, target)
+    os.makedirs(build_dir, exist_ok=True)
     inc, lib, abi = _torch_paths()
     py_inc = sysconfig.get_paths()["include"]
     header_deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     jobs_list = []
     objs = []
-    for f in sorted(os.listdir(CSRC)):
-        src = os.path.join(CSRC, f)
+    for f in sorted(os.listdir(src_dir)):
+        src = os.path.join(src_dir, f)
         if f.endswith(".hip"):
-            obj = os.path.join(BUILD, f[:-4] + ".o")
-            cmd = [HIPCC, *KERNEL_FLAGS, "-I", CSRC, "-c", src, "-o", obj]
+            obj = os.path.join(build_dir, f[:-4] + ".o")
+            cmd = [HIPCC, *KERNEL_FLAGS, *extra, "-I", CSRC, "-c", src, "-o", obj]
         elif f.endswith(".cpp"):
-            obj = os.path.join(BUILD, f[:-4] + ".o")
+            obj = os.path.join(build_dir, f[:-4] + ".o")
             cmd = [HIPCC, "-O2", "-fPIC", "-std=c++17", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
-                   "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H",
+                   f"-DTORCH_EXTENSION_NAME={name}", "-DTORCH_API_INCLUDE_EXTENSION_H",
                    f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-Wno-unused-result", "-Wno-deprecated-declarations",
                    *[f"-I{p}" for p in inc], f"-I{py_inc}", "-I", CSRC, "-c", src, "-o", obj]
         else:
@@ -81,7 +102,7 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
             for out in ex.map(_run, jobs_list):
                 if verbose and out.strip():
                     print(out)
-    target = target_path()
+    target = target_path(target)
     if _stale(target, objs):
         tmp = target + ".tmp"
         cmd = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp,

@@ -1,0 +1,294 @@
+// Python bindings of the ragged-step kernels (seqmix.hip): shape / dtype / device checks, outputs
+// from torch's caching allocator, launches on torch's current HIP stream.  Activations are fp32 or
+// bf16 (one flag per call, taken from the tensors); metadata tensors are int32 on the device.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <hip/hip_runtime.h>
+
+#include <optional>
+
+extern "C" {
+int edge_sm_embed(const int64_t* ids, const void* table, float* out, int rows, int W, int V, float scale, int f32,
+                  hipStream_t st);
+int edge_sm_scalar_norm(const float* x, const float* gain, void* y, int rows, int W, float eps, int f32, hipStream_t st);
+int edge_sm_relu2(const void* u, int ld, int c0, void* y, int rows, int C, int f32, hipStream_t st);
+int edge_sm_cat_cast(const float* a, const float* b, void* y, int rows, int W, int f32, hipStream_t st);
+int edge_sm_combine(float* x, const void* l, const void* r, const float* wl, const float* wr, const void* extra,
+                    int rows, int W, float eps, int f32, hipStream_t st);
+int edge_sm_gated_norm(const float* y, const void* z, int z_ld, const float* w, void* out, int rows, int C, int groups,
+                       float eps, int f32, hipStream_t st);
+int edge_sm_rope_write(const void* proj, int ld, const int* tok_seq, const int* tok_pos, const int* seq_slot,
+                       const int* ptab, int ptab_ld, const float* cs, void* q_out, void* kp, void* vp, int rows,
+                       int H, int G, int D, int Dv, int rot, int page, int f32, hipStream_t st);
+int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, const int* seq_slot,
+                        const int* seq_start, const int* seq_len, const int* ptab, int ptab_ld, int n, int max_blocks,
+                        int G, int D, int Dv, int page, int PB, int pool, int f32, hipStream_t st);
+int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
+                      const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
+                      int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
+                      int window, int pool, int f32, hipStream_t st);
+int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
+                      const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
+                      const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
+                      hipStream_t st);
+int edge_sm_ssd_scan(const void* xbc, int Cx, const void* u, int ld, int dt0, const float* dt_bias, const float* A_log,
+                     const float* Dp, float* state, const int* seq_slot, const int* seq_start, const int* seq_len,
+                     const int* seq_off, float* y, int n, int Hs, int P, int N, int groups, int f32, hipStream_t st);
+}
+
+namespace {
+
+hipStream_t stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+void check(int rc, const char* what) {
+  TORCH_CHECK(rc == 0, what, ": launch failed (", rc, rc > 0 ? std::string(": ") + hipGetErrorString((hipError_t)rc) : "",
+              ")");
+}
+
+bool is_act(const at::Tensor& t) { return t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16; }
+int f32(const at::Tensor& t) { return t.scalar_type() == at::kFloat ? 1 : 0; }
+at::ScalarType act_type(bool f) { return f ? at::kFloat : at::kBFloat16; }
+
+// a [rows, cols] view whose rows are contiguous (stride(1) == 1): returns the row stride
+int row_ld(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.dim() == 2 && (t.size(1) == 0 || t.stride(1) == 1), name, ": rows must be contiguous");
+  return (int)t.stride(0);
+}
+void chk_i32(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), name, ": int32 device tensor expected");
+}
+void chk_f32(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), name, ": fp32 device tensor expected");
+}
+void chk_table(const at::Tensor& ptab) {
+  TORCH_CHECK(ptab.is_cuda() && ptab.scalar_type() == at::kInt && ptab.dim() == 2 && ptab.stride(1) == 1,
+              "page table: int32 [slots, pages]");
+}
+
+at::Tensor sm_embed(const at::Tensor& ids, const at::Tensor& table, double scale) {
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kLong && ids.is_contiguous() && ids.dim() == 1, "ids: int64 [T]");
+  TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.is_contiguous() && is_act(table), "table: [V, W] fp32 / bf16");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(table.device());
+  auto out = at::empty({ids.size(0), table.size(1)}, table.options().dtype(at::kFloat));
+  check(edge_sm_embed(ids.data_ptr<int64_t>(), table.data_ptr(), out.data_ptr<float>(), (int)ids.size(0),
+                      (int)table.size(1), (int)table.size(0), (float)scale, f32(table), stream()), "sm_embed");
+  return out;
+}
+
+at::Tensor sm_scalar_norm(const at::Tensor& x, const at::Tensor& gain, double eps, bool out_f32) {
+  chk_f32(x, "x");
+  chk_f32(gain, "gain");
+  TORCH_CHECK(x.dim() == 2 && gain.numel() == 1, "x [T, W], gain [1]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  auto y = at::empty_like(x, x.options().dtype(act_type(out_f32)));
+  check(edge_sm_scalar_norm(x.data_ptr<float>(), gain.data_ptr<float>(), y.data_ptr(), (int)x.size(0), (int)x.size(1),
+                            (float)eps, out_f32, stream()), "sm_scalar_norm");
+  return y;
+}
+
+at::Tensor sm_relu2(const at::Tensor& u, int64_t c0, int64_t C) {
+  TORCH_CHECK(is_act(u), "u: fp32 / bf16");
+  const int ld = row_ld(u, "u");
+  TORCH_CHECK(c0 >= 0 && C >= 0 && c0 + C <= u.size(1), "columns out of range");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(u.device());
+  auto y = at::empty({u.size(0), C}, u.options());
+  check(edge_sm_relu2(u.data_ptr(), ld, (int)c0, y.data_ptr(), (int)u.size(0), (int)C, f32(u), stream()), "sm_relu2");
+  return y;
+}
+
+at::Tensor sm_cat_cast(const at::Tensor& a, const at::Tensor& b, bool out_f32) {
+  chk_f32(a, "a");
+  chk_f32(b, "b");
+  TORCH_CHECK(a.dim() == 2 && a.sizes() == b.sizes(), "a, b: fp32 [T, W]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  auto y = at::empty({a.size(0), 2 * a.size(1)}, a.options().dtype(act_type(out_f32)));
+  check(edge_sm_cat_cast(a.data_ptr<float>(), b.data_ptr<float>(), y.data_ptr(), (int)a.size(0), (int)a.size(1),
+                         out_f32, stream()), "sm_cat_cast");
+  return y;
+}
+
+void sm_combine(at::Tensor& x, const at::Tensor& l, const at::Tensor& r, const at::Tensor& wl, const at::Tensor& wr,
+                double eps, const std::optional<at::Tensor>& extra) {
+  chk_f32(x, "x");
+  chk_f32(wl, "wl");
+  chk_f32(wr, "wr");
+  TORCH_CHECK(x.dim() == 2 && l.sizes() == x.sizes() && r.sizes() == x.sizes() && l.is_contiguous() &&
+                  r.is_contiguous() && is_act(l) && r.scalar_type() == l.scalar_type() && l.is_cuda() && r.is_cuda(),
+              "left / right: [T, W] like x");
+  TORCH_CHECK(wl.numel() == x.size(1) && wr.numel() == x.size(1), "weights: [W]");
+  if (extra) TORCH_CHECK(extra->sizes() == x.sizes() && extra->is_contiguous() && extra->is_cuda() &&
+                             extra->scalar_type() == l.scalar_type(), "extra: [T, W] like left");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  check(edge_sm_combine(x.data_ptr<float>(), l.data_ptr(), r.data_ptr(), wl.data_ptr<float>(), wr.data_ptr<float>(),
+                        extra ? extra->data_ptr() : nullptr, (int)x.size(0), (int)x.size(1), (float)eps, f32(l),
+                        stream()), "sm_combine");
+}
+
+at::Tensor sm_gated_norm(const at::Tensor& y, const at::Tensor& z, const at::Tensor& w, int64_t groups, double eps,
+                         bool out_f32) {
+  chk_f32(y, "y");
+  chk_f32(w, "weight");
+  const int z_ld = row_ld(z, "z");
+  TORCH_CHECK(y.dim() == 2 && z.sizes() == y.sizes() && is_act(z) && f32(z) == (int)out_f32 && w.numel() == y.size(1),
+              "y fp32 [T, C], z [T, C] in the output dtype, weight [C]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(y.device());
+  auto out = at::empty_like(y, y.options().dtype(act_type(out_f32)));
+  check(edge_sm_gated_norm(y.data_ptr<float>(), z.data_ptr(), z_ld, w.data_ptr<float>(), out.data_ptr(), (int)y.size(0),
+                           (int)y.size(1), (int)groups, (float)eps, out_f32, stream()), "sm_gated_norm");
+  return out;
+}
+
+at::Tensor sm_rope_write(const at::Tensor& proj, const at::Tensor& tok_seq, const at::Tensor& tok_pos,
+                         const at::Tensor& seq_slot, const at::Tensor& ptab, const std::optional<at::Tensor>& rope,
+                         at::Tensor& kp, at::Tensor& vp, int64_t H, int64_t rot) {
+  const int ld = row_ld(proj, "proj");
+  chk_i32(tok_seq, "tok_seq");
+  chk_i32(tok_pos, "tok_pos");
+  chk_i32(seq_slot, "seq_slot");
+  chk_table(ptab);
+  TORCH_CHECK(is_act(proj) && kp.scalar_type() == proj.scalar_type() && vp.scalar_type() == proj.scalar_type() &&
+                  kp.is_cuda() && vp.is_cuda() && kp.is_contiguous() && vp.is_contiguous() && kp.dim() == 4 &&
+                  vp.dim() == 4, "pages: [pages, page, G, D] in proj's dtype");
+  const int64_t T = proj.size(0), page = kp.size(1), G = kp.size(2), D = kp.size(3), Dv = vp.size(3);
+  TORCH_CHECK(vp.size(0) == kp.size(0) && vp.size(1) == page && vp.size(2) == G, "k / v pages differ");
+  TORCH_CHECK(proj.size(1) == (H + G) * D + G * Dv, "proj: [T, (H + G) D + G Dv]");
+  TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T, "token metadata: [T]");
+  if (rot > 0) {
+    TORCH_CHECK(rope && rope->is_cuda() && rope->scalar_type() == at::kFloat && rope->is_contiguous() &&
+                    rope->dim() == 3 && rope->size(1) * 2 == rot && rope->size(2) == 2, "rope: fp32 [pos, rot/2, 2]");
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(proj.device());
+  auto q = at::empty({T, H, D}, proj.options());
+  check(edge_sm_rope_write(proj.data_ptr(), ld, tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(),
+                           seq_slot.data_ptr<int>(), ptab.data_ptr<int>(), (int)ptab.stride(0),
+                           rot > 0 ? rope->data_ptr<float>() : nullptr, q.data_ptr(), kp.data_ptr(), vp.data_ptr(), (int)T,
+                           (int)H, (int)G, (int)D, (int)Dv, (int)rot, (int)page, f32(proj), stream()), "sm_rope_write");
+  return q;
+}
+
+void sm_pool_blocks(const at::Tensor& kp, const at::Tensor& vp, at::Tensor& kb, at::Tensor& vb,
+                    const at::Tensor& seq_slot, const at::Tensor& seq_start, const at::Tensor& seq_len,
+                    const at::Tensor& ptab, int64_t pool, int64_t n, int64_t max_blocks) {
+  chk_i32(seq_slot, "seq_slot");
+  chk_i32(seq_start, "seq_start");
+  chk_i32(seq_len, "seq_len");
+  chk_table(ptab);
+  chk_f32(kb, "k_pool");
+  chk_f32(vb, "v_pool");
+  TORCH_CHECK(is_act(kp) && kp.is_cuda() && kp.is_contiguous() && vp.is_contiguous() && kp.dim() == 4 && vp.dim() == 4 &&
+                  vp.scalar_type() == kp.scalar_type(), "pages: [pages, page, G, D]");
+  const int64_t page = kp.size(1), G = kp.size(2), D = kp.size(3), Dv = vp.size(3);
+  TORCH_CHECK(pool > 0 && kb.dim() == 4 && kb.size(0) == kp.size(0) && kb.size(1) == (page + pool - 1) / pool &&
+                  kb.size(2) == G && kb.size(3) == D && vb.size(0) == kp.size(0) && vb.size(1) == kb.size(1) &&
+                  vb.size(2) == G && vb.size(3) == Dv, "pooled entries: [pages, ceil(page / pool), G, D]");
+  TORCH_CHECK(seq_slot.numel() >= n && seq_start.numel() >= n && seq_len.numel() >= n, "sequence metadata: [n]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(kp.device());
+  check(edge_sm_pool_blocks(kp.data_ptr(), vp.data_ptr(), kb.data_ptr<float>(), vb.data_ptr<float>(),
+                            seq_slot.data_ptr<int>(), seq_start.data_ptr<int>(), seq_len.data_ptr<int>(),
+                            ptab.data_ptr<int>(), (int)ptab.stride(0), (int)n, (int)max_blocks, (int)G, (int)D, (int)Dv,
+                            (int)page, (int)kb.size(1), (int)pool, f32(kp), stream()), "sm_pool_blocks");
+}
+
+at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& gate, const at::Tensor& kp,
+                        const at::Tensor& vp, const std::optional<at::Tensor>& kb, const std::optional<at::Tensor>& vb,
+                        const at::Tensor& tok_seq, const at::Tensor& tok_pos, const at::Tensor& seq_slot,
+                        const at::Tensor& ptab, double scale, int64_t window, int64_t pool, int64_t max_keys) {
+  chk_i32(tok_seq, "tok_seq");
+  chk_i32(tok_pos, "tok_pos");
+  chk_i32(seq_slot, "seq_slot");
+  chk_table(ptab);
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && is_act(q), "q: [T, H, D]");
+  TORCH_CHECK(kp.scalar_type() == q.scalar_type() && vp.scalar_type() == q.scalar_type() && kp.is_contiguous() &&
+                  vp.is_contiguous() && kp.dim() == 4 && vp.dim() == 4 && kp.size(3) == q.size(2), "pages: [pages, page, G, D]");
+  const int64_t T = q.size(0), H = q.size(1), D = q.size(2), page = kp.size(1), G = kp.size(2), Dv = vp.size(3);
+  TORCH_CHECK(max_keys <= ptab.size(1) * page, "page table too short for the step");
+  int gate_ld = 0, PB = 0;
+  if (gate) {
+    gate_ld = row_ld(*gate, "gate");
+    TORCH_CHECK(gate->size(0) == T && gate->size(1) == H && gate->scalar_type() == q.scalar_type(), "gate: [T, H]");
+  }
+  if (pool > 0 && window > 0) {
+    TORCH_CHECK(kb && vb, "pooled entries missing");
+    chk_f32(*kb, "k_pool");
+    chk_f32(*vb, "v_pool");
+    PB = (int)kb->size(1);
+    TORCH_CHECK(kb->size(0) == kp.size(0) && PB == (page + pool - 1) / pool && kb->size(2) == G && kb->size(3) == D &&
+                    vb->size(1) == PB && vb->size(3) == Dv, "pooled entries: [pages, ceil(page / pool), G, D]");
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  auto out = at::empty({T, H * Dv}, q.options());
+  check(edge_sm_attention(q.data_ptr(), gate ? gate->data_ptr() : nullptr, gate_ld, kp.data_ptr(), vp.data_ptr(),
+                          PB ? kb->data_ptr<float>() : nullptr, PB ? vb->data_ptr<float>() : nullptr,
+                          tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),
+                          ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)T, (int)H, (int)G, (int)D, (int)Dv,
+                          (int)page, PB, (float)scale, (int)window, PB ? (int)pool : 0, f32(q), stream()), "sm_attention");
+  return out;
+}
+
+at::Tensor sm_conv_silu(const at::Tensor& u, int64_t c0, int64_t C, const at::Tensor& w, const at::Tensor& bias,
+                        at::Tensor& state, const at::Tensor& tok_seq, const at::Tensor& tok_pos,
+                        const at::Tensor& seq_slot, const at::Tensor& seq_start, const at::Tensor& seq_len,
+                        const at::Tensor& seq_off, int64_t n) {
+  const int ld = row_ld(u, "u");
+  chk_f32(w, "conv weight");
+  chk_f32(bias, "conv bias");
+  for (const at::Tensor* t : {&tok_seq, &tok_pos, &seq_slot, &seq_start, &seq_len, &seq_off}) chk_i32(*t, "metadata");
+  const int64_t T = u.size(0), taps = w.size(1);
+  TORCH_CHECK(is_act(u) && c0 >= 0 && c0 + C <= u.size(1) && w.dim() == 2 && w.size(0) == C && bias.numel() == C,
+              "conv: weight [C, taps], bias [C], columns inside u");
+  TORCH_CHECK(state.is_cuda() && state.is_contiguous() && state.scalar_type() == u.scalar_type() && state.dim() == 3 &&
+                  state.size(1) == std::max<int64_t>(taps - 1, 1) && state.size(2) == C, "state: [slots, taps - 1, C]");
+  TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T && seq_slot.numel() >= n, "metadata sizes");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(u.device());
+  auto out = at::empty({T, C}, u.options());
+  check(edge_sm_conv_silu(u.data_ptr(), ld, (int)c0, (int)C, w.data_ptr<float>(), bias.data_ptr<float>(), state.data_ptr(),
+                          tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),
+                          seq_start.data_ptr<int>(), seq_len.data_ptr<int>(), seq_off.data_ptr<int>(), out.data_ptr(),
+                          (int)T, (int)n, (int)taps, f32(u), stream()), "sm_conv_silu");
+  return out;
+}
+
+at::Tensor sm_ssd_scan(const at::Tensor& xbc, const at::Tensor& u, int64_t dt0, const at::Tensor& dt_bias,
+                       const at::Tensor& A_log, const at::Tensor& D, at::Tensor& state, const at::Tensor& seq_slot,
+                       const at::Tensor& seq_start, const at::Tensor& seq_len, const at::Tensor& seq_off, int64_t n,
+                       int64_t Hs, int64_t P, int64_t N, int64_t groups) {
+  const int ld = row_ld(u, "u");
+  chk_f32(dt_bias, "dt_bias");
+  chk_f32(A_log, "A_log");
+  chk_f32(D, "D");
+  chk_f32(state, "state");
+  for (const at::Tensor* t : {&seq_slot, &seq_start, &seq_len, &seq_off}) chk_i32(*t, "metadata");
+  TORCH_CHECK(xbc.is_cuda() && xbc.is_contiguous() && xbc.dim() == 2 && is_act(xbc) &&
+                  xbc.scalar_type() == u.scalar_type() && xbc.size(1) == Hs * P + 2 * groups * N &&
+                  xbc.size(0) == u.size(0), "xbc: [T, inner + 2 groups N]");
+  TORCH_CHECK(dt0 >= 0 && dt0 + Hs <= u.size(1) && dt_bias.numel() == Hs && A_log.numel() == Hs && D.numel() == Hs,
+              "per-head constants: [heads]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == Hs && state.size(2) == N && state.size(3) == P,
+              "state: fp32 [slots, heads, N, vdim]");
+  TORCH_CHECK(seq_slot.numel() >= n && seq_start.numel() >= n && seq_len.numel() >= n && seq_off.numel() >= n,
+              "sequence metadata: [n]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(xbc.device());
+  auto y = at::empty({xbc.size(0), Hs * P}, xbc.options().dtype(at::kFloat));
+  check(edge_sm_ssd_scan(xbc.data_ptr(), (int)xbc.size(1), u.data_ptr(), ld, (int)dt0, dt_bias.data_ptr<float>(),
+                         A_log.data_ptr<float>(), D.data_ptr<float>(), state.data_ptr<float>(), seq_slot.data_ptr<int>(),
+                         seq_start.data_ptr<int>(), seq_len.data_ptr<int>(), seq_off.data_ptr<int>(), y.data_ptr<float>(),
+                         (int)n, (int)Hs, (int)P, (int)N, (int)groups, f32(xbc), stream()), "sm_ssd_scan");
+  return y;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("sm_embed", &sm_embed);
+  m.def("sm_scalar_norm", &sm_scalar_norm);
+  m.def("sm_relu2", &sm_relu2);
+  m.def("sm_cat_cast", &sm_cat_cast);
+  m.def("sm_combine", &sm_combine);
+  m.def("sm_gated_norm", &sm_gated_norm);
+  m.def("sm_rope_write", &sm_rope_write);
+  m.def("sm_pool_blocks", &sm_pool_blocks);
+  m.def("sm_attention", &sm_attention);
+  m.def("sm_conv_silu", &sm_conv_silu);
+  m.def("sm_ssd_scan", &sm_ssd_scan);
+}

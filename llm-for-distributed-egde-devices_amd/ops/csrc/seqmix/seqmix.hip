@@ -1,0 +1,561 @@
+// Kernels of the ragged-step sequence mixers (ops/seqmix.py): scalar-gain RMS norm, squared ReLU,
+// rotary + paged key / value write, block pooling, windowed attention with pooled blocks over a
+// paged cache, causal convolution with a per-slot tail, the Mamba-2 recurrence, the gated group
+// norm and the two-branch combine with the residual add.
+//
+// Every kernel is instantiated for fp32 and bf16 storage (template T); scores, softmax, norms,
+// decays and the recurrent state are fp32 in both.  A token is addressed by (sequence of the step,
+// position) and its key / value row by the sequence's page-table row, so a result does not depend
+// on how a prompt was cut into steps or on what else is in the batch: each query's visible keys are
+// walked in the same order from the same first key, each block mean sums its rows in position
+// order, and the recurrence steps token by token.
+#include "common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p) { return bf2f(*p); }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float siluf_(float x) { return x * sigmoidf_(x); }
+
+constexpr int NT = 256;
+
+// ---------------------------------------------------------------------------------- rows
+template <typename T>
+__global__ void __launch_bounds__(NT) embed_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
+                                                   float* __restrict__ out, int W, int V, float scale) {
+  const int t = blockIdx.x;
+  int64_t id = ids[t];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+  for (int c = threadIdx.x; c < W; c += NT) out[(size_t)t * W + c] = ldf<T>(table + (size_t)id * W + c) * scale;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(NT) scalar_norm_kernel(const float* __restrict__ x, const float* __restrict__ gain,
+                                                         T* __restrict__ y, int W, float eps) {
+  __shared__ float red[NT / 64];
+  const float* xr = x + (size_t)blockIdx.x * W;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += NT) { const float v = xr[c]; ss += v * v; }
+  ss = block_sum<NT>(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)W + eps) * gain[0];
+  for (int c = threadIdx.x; c < W; c += NT) stf<T>(y + (size_t)blockIdx.x * W + c, xr[c] * r);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(NT) relu2_kernel(const T* __restrict__ u, int ld, int c0, T* __restrict__ y, int C) {
+  const int t = blockIdx.x;
+  for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
+    const float v = fmaxf(ldf<T>(u + (size_t)t * ld + c0 + c), 0.f);
+    stf<T>(y + (size_t)t * C + c, v * v);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(NT) cat_cast_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                      T* __restrict__ y, int W) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < 2 * W; c += NT)
+    stf<T>(y + (size_t)t * 2 * W + c, c < W ? a[(size_t)t * W + c] : b[(size_t)t * W + c - W]);
+}
+
+// x += 0.5 (l / rms(l) * wl + r / rms(r) * wr) + extra
+template <typename T>
+__global__ void __launch_bounds__(NT) combine_kernel(float* __restrict__ x, const T* __restrict__ l,
+                                                     const T* __restrict__ r, const float* __restrict__ wl,
+                                                     const float* __restrict__ wr, const T* __restrict__ extra, int W,
+                                                     float eps) {
+  __shared__ float red[NT / 64];
+  const size_t row = (size_t)blockIdx.x * W;
+  float sl = 0.f, sr = 0.f;
+  for (int c = threadIdx.x; c < W; c += NT) {
+    const float a = ldf<T>(l + row + c), b = ldf<T>(r + row + c);
+    sl += a * a;
+    sr += b * b;
+  }
+  sl = block_sum<NT>(sl, red);
+  sr = block_sum<NT>(sr, red);
+  const float rl = 1.f / sqrtf(sl / (float)W + eps), rr = 1.f / sqrtf(sr / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += NT) {
+    float v = 0.5f * (ldf<T>(l + row + c) * rl * wl[c] + ldf<T>(r + row + c) * rr * wr[c]);
+    if (extra) v += ldf<T>(extra + row + c);
+    x[row + c] += v;
+  }
+}
+
+// out = (y silu(z)) / rms over each of `groups` equal parts * w
+template <typename T>
+__global__ void __launch_bounds__(NT) gated_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int z_ld,
+                                                        const float* __restrict__ w, T* __restrict__ out, int C,
+                                                        int groups, float eps) {
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x, g = blockIdx.y, gs = C / groups;
+  const float* yr = y + (size_t)t * C + g * gs;
+  const T* zr = z + (size_t)t * z_ld + g * gs;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < gs; c += NT) {
+    const float v = yr[c] * siluf_(ldf<T>(zr + c));
+    ss += v * v;
+  }
+  ss = block_sum<NT>(ss, red);
+  const float r = 1.f / sqrtf(ss / (float)gs + eps);
+  for (int c = threadIdx.x; c < gs; c += NT)
+    stf<T>(out + (size_t)t * C + g * gs + c, yr[c] * siluf_(ldf<T>(zr + c)) * r * w[g * gs + c]);
+}
+
+// ---------------------------------------------------------------------------------- rotary + paged write
+// proj row = q [H, D] | k [G, D] | v [G, Dv]; cs [positions, rot / 2, 2]
+template <typename T>
+__global__ void __launch_bounds__(NT) rope_write_kernel(const T* __restrict__ proj, int ld, const int* __restrict__ tok_seq,
+                                                        const int* __restrict__ tok_pos, const int* __restrict__ seq_slot,
+                                                        const int* __restrict__ ptab, int ptab_ld,
+                                                        const float* __restrict__ cs, T* __restrict__ q_out,
+                                                        T* __restrict__ kp, T* __restrict__ vp, int H, int G, int D, int Dv,
+                                                        int rot, int page) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t], slot = seq_slot[tok_seq[t]];
+  const size_t prow = (size_t)ptab[(size_t)slot * ptab_ld + pos / page] * page + pos % page;
+  const T* row = proj + (size_t)t * ld;
+  const int half = rot >> 1, nqk = (H + G) * D;
+  const float* c = cs ? cs + (size_t)pos * rot : nullptr;          // rot / 2 pairs of (cos, sin)
+  for (int e = threadIdx.x; e < nqk; e += NT) {
+    const int hh = e / D, d = e % D;
+    float v = ldf<T>(row + e);
+    if (d < rot) {
+      const int i = d < half ? d : d - half;
+      const float co = c[2 * i], si = c[2 * i + 1];
+      const float o = ldf<T>(row + (d < half ? e + half : e - half));
+      v = d < half ? v * co - o * si : v * co + o * si;
+    }
+    if (hh < H) stf<T>(q_out + (size_t)t * H * D + e, v);
+    else stf<T>(kp + (prow * G + (hh - H)) * D + d, v);
+  }
+  for (int e = threadIdx.x; e < G * Dv; e += NT) vp[prow * G * Dv + e] = row[nqk + e];
+}
+
+// mean over the rows of each block whose last token lies in [start, start + len)
+template <typename T>
+__global__ void __launch_bounds__(NT) pool_kernel(const T* __restrict__ kp, const T* __restrict__ vp,
+                                                  float* __restrict__ kb, float* __restrict__ vb,
+                                                  const int* __restrict__ seq_slot, const int* __restrict__ seq_start,
+                                                  const int* __restrict__ seq_len, const int* __restrict__ ptab,
+                                                  int ptab_ld, int G, int D, int Dv, int page, int PB, int pool) {
+  const int s = blockIdx.x;
+  const int start = seq_start[s], end = start + seq_len[s];
+  const int b = start / pool + blockIdx.y;
+  if (b * pool + pool - 1 >= end) return;
+  const int* pt = ptab + (size_t)seq_slot[s] * ptab_ld;
+  const int p0 = b * pool;
+  const size_t dst = (size_t)pt[p0 / page] * PB + (p0 % page) / pool;
+  const float inv = 1.f / (float)pool;
+  const int nk = G * D, nv = G * Dv;
+  for (int e = threadIdx.x; e < nk + nv; e += NT) {
+    float acc = 0.f;
+    for (int j = 0; j < pool; ++j) {
+      const int p = p0 + j;
+      const size_t r = (size_t)pt[p / page] * page + p % page;
+      acc += e < nk ? ldf<T>(kp + r * nk + e) : ldf<T>(vp + r * nv + (e - nk));
+    }
+    if (e < nk) kb[dst * nk + e] = acc * inv;
+    else vb[dst * nv + (e - nk)] = acc * inv;
+  }
+}
+
+// ---------------------------------------------------------------------------------- attention
+// One workgroup per (token, kv head): its R = H / G query heads share every key / value row read.
+// Keys are walked in chunks of KC: (A) thread j scores key j against the R queries (q in LDS,
+// broadcast reads), (B) wave w keeps the running max / sum of heads w, w + 4, .. and turns the
+// chunk's scores into weights, (C) wave w accumulates weight x value over its quarter of the
+// chunk with lane = value coordinate (coalesced row reads).  Tokens of the window first, then the
+// pooled blocks (fp32 rows): one softmax over both.
+constexpr int KC = 256;
+
+template <typename KT, int RMAX, int DVL>
+__device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const KT* __restrict__ vbase, int cnt, int g,
+                                           int G, int D, int Dv, int R, const float* q_s, float* s_s, int* row_s,
+                                           float* m_s, float* l_s, float* a_s, int rowidx, float (&acc)[RMAX][DVL]) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (A) scores
+  {
+    float a[RMAX];
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) a[r] = 0.f;
+    if (tid < cnt) {
+      const KT* kr = kbase + ((size_t)rowidx * G + g) * D;
+      for (int d = 0; d < D; ++d) {
+        const float kv = ldf<KT>(kr + d);
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) a[r] += q_s[r * D + d] * kv;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) s_s[r * KC + tid] = tid < cnt ? a[r] : -INFINITY;
+    row_s[tid] = rowidx;
+  }
+  __syncthreads();
+  // (B) running softmax statistics, one head per wave at a time
+  for (int r = wave; r < R; r += NT / 64) {
+    float v[KC / 64], cm = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < KC / 64; ++k) { v[k] = s_s[r * KC + lane + 64 * k]; cm = fmaxf(cm, v[k]); }
+    cm = wave_max(cm);
+    const float mo = m_s[r], mn = fmaxf(mo, cm);
+    float ls = 0.f;
+#pragma unroll
+    for (int k = 0; k < KC / 64; ++k) {
+      const float p = expf(v[k] - mn);
+      s_s[r * KC + lane + 64 * k] = p;
+      ls += p;
+    }
+    ls = wave_sum(ls);
+    if (lane == 0) {
+      const float al = expf(mo - mn);                      // mo = -inf on the first chunk: 0
+      m_s[r] = mn;
+      l_s[r] = l_s[r] * al + ls;
+      a_s[r] = al;
+    }
+  }
+  __syncthreads();
+  // (C) weights x values
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r) {
+    const float al = r < R ? a_s[r] : 1.f;
+#pragma unroll
+    for (int dl = 0; dl < DVL; ++dl) acc[r][dl] *= al;
+  }
+  const int j1 = min(cnt, 64 * (wave + 1));
+  for (int j = 64 * wave; j < j1; ++j) {
+    const KT* vr = vbase + ((size_t)row_s[j] * G + g) * Dv;
+    float vv[DVL];
+#pragma unroll
+    for (int dl = 0; dl < DVL; ++dl) vv[dl] = lane + 64 * dl < Dv ? ldf<KT>(vr + lane + 64 * dl) : 0.f;
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+      const float p = s_s[r * KC + j];
+#pragma unroll
+      for (int dl = 0; dl < DVL; ++dl) acc[r][dl] += p * vv[dl];
+    }
+  }
+  __syncthreads();
+}
+
+template <typename T, int RMAX, int DVL>
+__global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const T* __restrict__ gate, int gate_ld,
+                                                  const T* __restrict__ kp, const T* __restrict__ vp,
+                                                  const float* __restrict__ kb, const float* __restrict__ vb,
+                                                  const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                                  const int* __restrict__ seq_slot, const int* __restrict__ ptab,
+                                                  int ptab_ld, T* __restrict__ out, int H, int G, int D, int Dv,
+                                                  int page, int PB, float scale, int window, int pool) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int t = blockIdx.x, g = blockIdx.y, R = H / G;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* q_s = smem;                         // [RMAX][D]
+  float* s_s = q_s + RMAX * D;               // [RMAX][KC]
+  float* red = s_s + RMAX * KC;              // [RMAX][Dv]
+  float* m_s = red + RMAX * Dv;              // [RMAX] x 3
+  float* l_s = m_s + RMAX;
+  float* a_s = l_s + RMAX;
+  int* row_s = reinterpret_cast<int*>(a_s + RMAX);   // [KC]
+  const int i = tok_pos[t];
+  const int* pt = ptab + (size_t)seq_slot[tok_seq[t]] * ptab_ld;
+  for (int e = tid; e < RMAX * D; e += NT) {
+    const int r = e / D, d = e % D;
+    q_s[e] = r < R ? ldf<T>(q + ((size_t)t * H + g * R + r) * D + d) * scale : 0.f;
+  }
+  for (int e = tid; e < RMAX * Dv; e += NT) red[e] = 0.f;
+  if (tid < RMAX) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; }
+  float acc[RMAX][DVL];
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+    for (int dl = 0; dl < DVL; ++dl) acc[r][dl] = 0.f;
+  __syncthreads();
+  const int jlo = window > 0 ? max(0, i - window + 1) : 0;
+  const int nt = i - jlo + 1;
+  const int nb = (window > 0 && pool > 0 && i - window + 1 > 0) ? (i - window + 1) / pool : 0;
+  for (int c0 = 0; c0 < nt; c0 += KC) {
+    const int j = jlo + c0 + tid;
+    const int rowidx = c0 + tid < nt ? pt[j / page] * page + j % page : 0;
+    attn_chunk<T, RMAX, DVL>(kp, vp, min(KC, nt - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
+  }
+  for (int c0 = 0; c0 < nb; c0 += KC) {
+    const int p0 = (c0 + tid) * pool;
+    const int rowidx = c0 + tid < nb ? pt[p0 / page] * PB + (p0 % page) / pool : 0;
+    attn_chunk<float, RMAX, DVL>(kb, vb, min(KC, nb - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
+  }
+  // sum the four waves' partial outputs, normalise, gate
+  for (int w = 0; w < NT / 64; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+        for (int dl = 0; dl < DVL; ++dl)
+          if (r < R && lane + 64 * dl < Dv) red[r * Dv + lane + 64 * dl] += acc[r][dl];
+    }
+    __syncthreads();
+  }
+  for (int e = tid; e < R * Dv; e += NT) {
+    const int r = e / Dv, h = g * R + r;
+    float o = red[e] / l_s[r];
+    if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + h));
+    stf<T>(out + ((size_t)t * H + h) * Dv + e % Dv, o);
+  }
+}
+
+// ---------------------------------------------------------------------------------- convolution
+constexpr int MAX_TAPS = 16;
+
+template <typename T>
+__global__ void __launch_bounds__(NT) conv_kernel(const T* __restrict__ u, int ld, int c0, int C,
+                                                  const float* __restrict__ w, const float* __restrict__ bias,
+                                                  const T* __restrict__ state, const int* __restrict__ tok_seq,
+                                                  const int* __restrict__ tok_pos, const int* __restrict__ seq_slot,
+                                                  const int* __restrict__ seq_start, const int* __restrict__ seq_off,
+                                                  T* __restrict__ out, int taps) {
+  const int t = blockIdx.x, s = tok_seq[t];
+  const int pos = tok_pos[t], start = seq_start[s], off = seq_off[s];
+  const T* st = state + (size_t)seq_slot[s] * (taps - 1) * C;
+  for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
+    float acc = bias[c];
+    for (int k = 0; k < taps; ++k) {
+      const int p = pos - (taps - 1) + k;
+      float x = 0.f;
+      if (p >= start) x = ldf<T>(u + (size_t)(off + p - start) * ld + c0 + c);
+      else if (p >= 0) x = ldf<T>(st + (size_t)(p - (start - (taps - 1))) * C + c);
+      acc += w[c * taps + k] * x;
+    }
+    stf<T>(out + (size_t)t * C + c, siluf_(acc));
+  }
+}
+
+// the inputs of each sequence's last taps - 1 positions, in position order
+template <typename T>
+__global__ void __launch_bounds__(NT) conv_state_kernel(const T* __restrict__ u, int ld, int c0, int C,
+                                                        T* __restrict__ state, const int* __restrict__ seq_slot,
+                                                        const int* __restrict__ seq_start,
+                                                        const int* __restrict__ seq_len, const int* __restrict__ seq_off,
+                                                        int taps) {
+  const int s = blockIdx.x;
+  const int start = seq_start[s], end = start + seq_len[s], off = seq_off[s];
+  T* st = state + (size_t)seq_slot[s] * (taps - 1) * C;
+  for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
+    T keep[MAX_TAPS];
+#pragma unroll
+    for (int k = 0; k < MAX_TAPS; ++k) {
+      if (k < taps - 1) {
+        const int p = end - (taps - 1) + k;
+        T v = T(0);                                       // bit pattern 0 = 0.0 in both storage types
+        if (p >= start) v = u[(size_t)(off + p - start) * ld + c0 + c];
+        else if (p >= 0) v = st[(size_t)(p - (start - (taps - 1))) * C + c];
+        keep[k] = v;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < MAX_TAPS; ++k)
+      if (k < taps - 1) st[(size_t)k * C + c] = keep[k];
+  }
+}
+
+// ---------------------------------------------------------------------------------- state-space recurrence
+// One wave per (sequence, head, 64 value columns); lane = column p holds S[0..N)[p] in registers.
+// Tokens are staged TC at a time (B, C rows, step size and decay in LDS), then stepped in order.
+constexpr int TC = 16;
+
+template <typename T, int NMAX>
+__global__ void __launch_bounds__(64) ssd_kernel(const T* __restrict__ xbc, int Cx, const T* __restrict__ u, int ld,
+                                                 int dt0, const float* __restrict__ dt_bias,
+                                                 const float* __restrict__ A_log, const float* __restrict__ Dp,
+                                                 float* __restrict__ state, const int* __restrict__ seq_slot,
+                                                 const int* __restrict__ seq_start, const int* __restrict__ seq_len,
+                                                 const int* __restrict__ seq_off, float* __restrict__ y, int Hs, int P,
+                                                 int N, int groups) {
+  __shared__ float B_s[TC][NMAX], C_s[TC][NMAX], dt_s[TC], dec_s[TC];
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, p = blockIdx.z * 64 + tid;
+  const int start = seq_start[s], len = seq_len[s], off = seq_off[s];
+  const int g = h / (Hs / groups), inner = Hs * P;
+  float* st = state + ((size_t)seq_slot[s] * Hs + h) * N * P;
+  float S[NMAX];
+#pragma unroll
+  for (int n = 0; n < NMAX; ++n) S[n] = (start > 0 && n < N && p < P) ? st[(size_t)n * P + p] : 0.f;
+  const float a = expf(A_log[h]), Dh = Dp[h], bias = dt_bias[h];
+  for (int t0 = 0; t0 < len; t0 += TC) {
+    const int tc = min(TC, len - t0);
+    __syncthreads();
+    for (int e = tid; e < tc * NMAX; e += 64) {
+      const int tt = e / NMAX, n = e % NMAX;
+      const T* row = xbc + (size_t)(off + t0 + tt) * Cx + inner + g * N;
+      B_s[tt][n] = n < N ? ldf<T>(row + n) : 0.f;
+      C_s[tt][n] = n < N ? ldf<T>(row + groups * N + n) : 0.f;
+    }
+    if (tid < tc) {
+      const float raw = ldf<T>(u + (size_t)(off + t0 + tid) * ld + dt0 + h) + bias;
+      const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+      dt_s[tid] = dt;
+      dec_s[tid] = expf(-a * dt);
+    }
+    __syncthreads();
+    if (p < P) {
+      for (int tt = 0; tt < tc; ++tt) {
+        const size_t row = (size_t)(off + t0 + tt);
+        const float xv = ldf<T>(xbc + row * Cx + h * P + p);
+        const float dx = dt_s[tt] * xv, dec = dec_s[tt];
+        float yv = 0.f;
+#pragma unroll
+        for (int n = 0; n < NMAX; ++n) {
+          S[n] = dec * S[n] + B_s[tt][n] * dx;
+          yv += S[n] * C_s[tt][n];
+        }
+        y[row * inner + h * P + p] = yv + Dh * xv;
+      }
+    }
+  }
+  if (p < P) {
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+      if (n < N) st[(size_t)n * P + p] = S[n];
+  }
+}
+
+}  // namespace
+
+#define SM_T(f32, ...)                                  \
+  do {                                                  \
+    if (f32) { using T = float; __VA_ARGS__; }          \
+    else { using T = bf16_t; __VA_ARGS__; }             \
+  } while (0)
+
+extern "C" {
+
+int edge_sm_embed(const int64_t* ids, const void* table, float* out, int rows, int W, int V, float scale, int f32,
+                  hipStream_t st) {
+  if (rows == 0) return 0;
+  SM_T(f32, hipLaunchKernelGGL(embed_kernel<T>, dim3(rows), dim3(NT), 0, st, ids, (const T*)table, out, W, V, scale));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_scalar_norm(const float* x, const float* gain, void* y, int rows, int W, float eps, int f32,
+                        hipStream_t st) {
+  if (rows == 0) return 0;
+  SM_T(f32, hipLaunchKernelGGL(scalar_norm_kernel<T>, dim3(rows), dim3(NT), 0, st, x, gain, (T*)y, W, eps));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_relu2(const void* u, int ld, int c0, void* y, int rows, int C, int f32, hipStream_t st) {
+  if (rows == 0 || C == 0) return 0;
+  const int gy = (C + NT * 4 - 1) / (NT * 4);
+  SM_T(f32, hipLaunchKernelGGL(relu2_kernel<T>, dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, (T*)y, C));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_cat_cast(const float* a, const float* b, void* y, int rows, int W, int f32, hipStream_t st) {
+  if (rows == 0) return 0;
+  SM_T(f32, hipLaunchKernelGGL(cat_cast_kernel<T>, dim3(rows), dim3(NT), 0, st, a, b, (T*)y, W));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_combine(float* x, const void* l, const void* r, const float* wl, const float* wr, const void* extra,
+                    int rows, int W, float eps, int f32, hipStream_t st) {
+  if (rows == 0) return 0;
+  SM_T(f32, hipLaunchKernelGGL(combine_kernel<T>, dim3(rows), dim3(NT), 0, st, x, (const T*)l, (const T*)r, wl, wr,
+                               (const T*)extra, W, eps));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_gated_norm(const float* y, const void* z, int z_ld, const float* w, void* out, int rows, int C, int groups,
+                       float eps, int f32, hipStream_t st) {
+  if (rows == 0) return 0;
+  if (groups <= 0 || C % groups) return -2;
+  SM_T(f32, hipLaunchKernelGGL(gated_norm_kernel<T>, dim3(rows, groups), dim3(NT), 0, st, y, (const T*)z, z_ld, w,
+                               (T*)out, C, groups, eps));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_rope_write(const void* proj, int ld, const int* tok_seq, const int* tok_pos, const int* seq_slot,
+                       const int* ptab, int ptab_ld, const float* cs, void* q_out, void* kp, void* vp, int rows,
+                       int H, int G, int D, int Dv, int rot, int page, int f32, hipStream_t st) {
+  if (rows == 0) return 0;
+  if (rot % 2 || rot > D || (rot > 0 && !cs)) return -2;
+  SM_T(f32, hipLaunchKernelGGL(rope_write_kernel<T>, dim3(rows), dim3(NT), 0, st, (const T*)proj, ld, tok_seq, tok_pos,
+                               seq_slot, ptab, ptab_ld, cs, (T*)q_out, (T*)kp, (T*)vp, H, G, D, Dv, rot, page));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, const int* seq_slot,
+                        const int* seq_start, const int* seq_len, const int* ptab, int ptab_ld, int n, int max_blocks,
+                        int G, int D, int Dv, int page, int PB, int pool, int f32, hipStream_t st) {
+  if (n == 0 || max_blocks <= 0) return 0;
+  SM_T(f32, hipLaunchKernelGGL(pool_kernel<T>, dim3(n, max_blocks), dim3(NT), 0, st, (const T*)kp, (const T*)vp, kb, vb,
+                               seq_slot, seq_start, seq_len, ptab, ptab_ld, G, D, Dv, page, PB, pool));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
+                      const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
+                      int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
+                      int window, int pool, int f32, hipStream_t st) {
+  if (rows == 0) return 0;
+  if (G <= 0 || H % G || Dv > 256 || H / G > 16) return -2;
+  const int R = H / G;
+  const int rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16;
+  const size_t lds = sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 3 * rmax) +
+                     sizeof(int) * KC;
+  if (lds > 64 * 1024) return -3;
+#define SM_ATT(RM, DL)                                                                                              \
+  SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL>), dim3(rows, G), dim3(NT), lds, st, (const T*)q,            \
+                               (const T*)gate, gate_ld, (const T*)kp, (const T*)vp, kb, vb, tok_seq, tok_pos,       \
+                               seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool))
+#define SM_ATT_R(DL)                 \
+  switch (rmax) {                    \
+    case 1: SM_ATT(1, DL); break;    \
+    case 2: SM_ATT(2, DL); break;    \
+    case 4: SM_ATT(4, DL); break;    \
+    case 8: SM_ATT(8, DL); break;    \
+    default: SM_ATT(16, DL); break;  \
+  }
+  if (Dv <= 128) { SM_ATT_R(2); }
+  else { SM_ATT_R(4); }
+#undef SM_ATT_R
+#undef SM_ATT
+  return (int)hipGetLastError();
+}
+
+int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
+                      const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
+                      const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
+                      hipStream_t st) {
+  if (rows == 0) return 0;
+  if (taps < 1 || taps > MAX_TAPS) return -2;
+  const int gy = (C + NT - 1) / NT;
+  SM_T(f32, hipLaunchKernelGGL(conv_kernel<T>, dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, w, bias,
+                               (const T*)state, tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps));
+  if (taps > 1)
+    SM_T(f32, hipLaunchKernelGGL(conv_state_kernel<T>, dim3(n, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, (T*)state,
+                                 seq_slot, seq_start, seq_len, seq_off, taps));
+  return (int)hipGetLastError();
+}
+
+int edge_sm_ssd_scan(const void* xbc, int Cx, const void* u, int ld, int dt0, const float* dt_bias, const float* A_log,
+                     const float* Dp, float* state, const int* seq_slot, const int* seq_start, const int* seq_len,
+                     const int* seq_off, float* y, int n, int Hs, int P, int N, int groups, int f32, hipStream_t st) {
+  if (n == 0) return 0;
+  if (N > 256 || groups <= 0 || Hs % groups) return -2;
+  const dim3 grid(n, Hs, (P + 63) / 64);
+#define SM_SSD(NM)                                                                                                  \
+  SM_T(f32, hipLaunchKernelGGL((ssd_kernel<T, NM>), grid, dim3(64), 0, st, (const T*)xbc, Cx, (const T*)u, ld, dt0, \
+                               dt_bias, A_log, Dp, state, seq_slot, seq_start, seq_len, seq_off, y, Hs, P, N, groups))
+  if (N <= 16) SM_SSD(16);
+  else if (N <= 32) SM_SSD(32);
+  else if (N <= 64) SM_SSD(64);
+  else if (N <= 128) SM_SSD(128);
+  else SM_SSD(256);
+#undef SM_SSD
+  return (int)hipGetLastError();
+}
+
+}  // extern "C"

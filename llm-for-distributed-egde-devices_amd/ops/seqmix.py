@@ -29,8 +29,31 @@ def _gpu(t: torch.Tensor) -> bool:
     return _ops().gpu_path(t)
 
 
+_EXT = None
+
+
 def _ext():
-    return _ops().ext()
+    """The ragged-step kernel library (``ops/_seqmix*.so``, built from ``csrc/seqmix`` on first use
+    when absent; a failed build or import raises: GPU tensors never fall back to the PyTorch forms)."""
+    global _EXT
+    if _EXT is None:
+        import importlib
+        name = __name__.rsplit(".", 1)[0] + "._seqmix"
+        try:
+            _EXT = importlib.import_module(name)
+        except ImportError:
+            from . import build
+            build.build(targets=("seqmix",))
+            importlib.invalidate_caches()
+            _EXT = importlib.import_module(name)
+    return _EXT
+
+
+def available() -> bool:
+    try:
+        return _ext() is not None
+    except Exception:  # noqa: BLE001
+        return False
 
 
 @dataclass
