@@ -99,6 +99,12 @@ def parse(argv=None):
                     help="chunked prefill size with HeadInfer (default: the whole prompt in one chunk)")
     ap.add_argument("--headinfer-heads", type=int, default=None,
                     help="HeadInfer: KV heads per layer kept on the GPU, the rest offloaded to pinned host memory")
+    ap.add_argument("--hybrid-compare", action="store_true",
+                    help="instead of the headline workload: prefill / decode throughput of the Nudadra layer-spec "
+                         "model beside the parallel-residual decoder of equal size (one JSON line)")
+    ap.add_argument("--hybrid-sizes", default="w1024,w2048", help="comma list of w1024 | w2048 | w4096")
+    ap.add_argument("--hybrid-prompt", type=int, default=4096)
+    ap.add_argument("--hybrid-batch", type=int, default=4)
     ap.add_argument("--metrics-out", default=os.environ.get("EDGELLM_METRICS"),
                     help="append the result record (plus HBM peak) to this JSONL file")
     return ap.parse_args(argv)
@@ -429,6 +435,12 @@ def launch_ranks(n: int, argv) -> int:
 def main(argv=None):
     raw = list(sys.argv[1:] if argv is None else argv)
     args = parse(raw)
+    if args.hybrid_compare:
+        from edgellm.engine import ragged_bench
+        out = ragged_bench.run(args.hybrid_sizes.split(","), args.hybrid_prompt, args.hybrid_batch, args.steps,
+                               args.device)
+        print(json.dumps(out), flush=True)
+        return out
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # no torchrun around us: start the N rank processes ourselves (the parent stays GPU-free)
         raise SystemExit(launch_ranks(args.gpus, raw))

@@ -1,0 +1,167 @@
+"""Prefill / decode throughput of a layer-spec (Nudadra) model beside the closest row-cache model
+of equal size (``bench.py --hybrid-compare``).
+
+Sizes resemble real layers (random weights): the hybrid layer has windowed attention with pooled
+blocks + a Mamba-2 mixer + a squared-ReLU feed-forward; the comparison model is the
+parallel-residual decoder (Phi layout: one norm, attention and MLP side by side) with the same
+width, layer count, attention heads, head size, feed-forward width and vocabulary, bf16.
+
+Per size: prefill tokens/s of one prompt of ``prompt`` tokens, decode tokens/s and ms/step of
+``batch`` sequences at that context, and per-op times of one prefill and one decode step of the
+hybrid (device events around each ``ops.seqmix`` call) with the bytes / flops each moves, so an op
+can be priced against the 8 TB/s / 2.5 PFLOP/s roofline.
+"""
+from __future__ import annotations
+
+import time
+from typing import Dict, List
+
+import torch
+
+from ..models.configs import LayerSpec, ModelConfig, SSDSpec, WindowAttnSpec, PRESETS
+from ..models.decoder import build_model
+from ..models.hybrid import build_hybrid
+from .generate import Generator, SamplingParams
+from .ragged import RaggedEngine
+
+SIZES = {
+    "w1024": dict(width=1024, layers=4, heads=16, kv=4, dim=64, window=512, pool=16, s_heads=16, s_vdim=64, state=64,
+                  ff=4096, vocab=32000),
+    "w2048": dict(width=2048, layers=4, heads=16, kv=4, dim=128, window=1024, pool=32, s_heads=32, s_vdim=64,
+                  state=128, ff=8192, vocab=32000),
+    "w4096": dict(width=4096, layers=2, heads=32, kv=8, dim=128, window=2048, pool=64, s_heads=64, s_vdim=64,
+                  state=128, ff=14336, vocab=32000),
+}
+
+
+def hybrid_config(s: dict) -> ModelConfig:
+    a = WindowAttnSpec(s["heads"], s["kv"], s["dim"], s["dim"], s["dim"] ** -0.5, s["window"], s["pool"], s["dim"],
+                       500000.0, {"rope_type": "yarn", "factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0})
+    m = SSDSpec(s["s_heads"], s["s_vdim"], s["state"], 1, 4, 1)
+    specs = [LayerSpec("parallel", a, m, s["ff"]) for _ in range(s["layers"])]
+    return ModelConfig(arch="nudadra", vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
+                       num_heads=s["heads"], num_kv_heads=s["kv"], intermediate_size=s["ff"], head_dim=s["dim"],
+                       max_position_embeddings=1 << 20, norm="rms_scalar", norm_eps=1e-6, act="relu2",
+                       parallel_residual=True, shared_input_norm=True, name="nudadra-bench", layer_specs=specs,
+                       embed_scale=1.0)
+
+
+def closest_config(s: dict) -> ModelConfig:
+    return PRESETS["phi-2"].replace(vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
+                                    num_heads=s["heads"], num_kv_heads=s["kv"], head_dim=s["dim"], rotary_dim=s["dim"],
+                                    intermediate_size=s["ff"], max_position_embeddings=1 << 16, name="phi-layout")
+
+
+def _timed(fn, reps: int, warm: int = 1) -> float:
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def bench_hybrid(s: dict, prompt: int, batch: int, steps: int, device) -> Dict:
+    model = build_hybrid(hybrid_config(s), torch.bfloat16, device, seed=0)
+    ids = torch.randint(0, s["vocab"], (prompt,), generator=torch.Generator().manual_seed(0)).tolist()
+    page = 64
+    eng = RaggedEngine(model, (batch + 1) * ((prompt + steps + 2 * page) // page) * page, slots=batch + 1)
+
+    def prefill():
+        eng.step([("p", ids, [prompt - 1])])
+        eng.close("p")
+    t_pre = _timed(prefill, 3)
+    for b in range(batch):
+        eng.step([(b, ids, [prompt - 1])])
+    tok = [1] * batch
+    dec = lambda: eng.step([(b, [tok[b]], [0]) for b in range(batch)])
+    t_dec = _timed(dec, steps, warm=3)
+    out = {"prefill_tok_s": prompt / t_pre, "prefill_ms": t_pre * 1e3, "decode_tok_s": batch / t_dec,
+           "decode_ms_per_step": t_dec * 1e3, "decode_graph": bool(getattr(eng, "graphs_used", False)),
+           "ops_prefill_us": op_times(eng, [("q", ids, [prompt - 1])], close=["q"]),
+           "ops_decode_us": op_times(eng, [(b, [tok[b]], [0]) for b in range(batch)])}
+    return out
+
+
+def op_times(eng: RaggedEngine, entries, close=()) -> Dict[str, float]:
+    """Device time per op kind over one step (sum over layers), from events around every
+    ``ops.seqmix`` call and every projection (eager step: no graph)."""
+    from ..ops import seqmix
+    import torch.nn.functional as F
+    marks: List[tuple] = []
+    names = ["embedding_scaled", "scalar_rms_norm", "relu2", "cat_cast", "combine_residual", "gated_group_norm",
+             "rope_paged_write", "pool_blocks", "window_pool_attention", "conv_silu", "ssd_scan", "linear_f32"]
+    saved = {n: getattr(seqmix, n) for n in names}
+    lin = F.linear
+
+    def wrap(name, fn):
+        def inner(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **k)
+            e1.record()
+            marks.append((name, e0, e1))
+            return r
+        return inner
+    graphs = getattr(eng, "use_graphs", None)
+    try:
+        if graphs is not None:
+            eng.use_graphs = False
+        for n in names:
+            setattr(seqmix, n, wrap(n, saved[n]))
+        from ..models import layers as L
+        orig_fwd = L.Linear.forward
+        L.Linear.forward = wrap("projections", orig_fwd)
+        eng.step(entries)
+        torch.cuda.synchronize()
+    finally:
+        for n in names:
+            setattr(seqmix, n, saved[n])
+        L.Linear.forward = orig_fwd
+        if graphs is not None:
+            eng.use_graphs = graphs
+    for r in close:
+        eng.close(r)
+    out: Dict[str, float] = {}
+    for name, e0, e1 in marks:
+        out[name] = out.get(name, 0.0) + e0.elapsed_time(e1) * 1e3
+    return {k: round(v, 1) for k, v in out.items()}
+
+
+def bench_closest(s: dict, prompt: int, batch: int, steps: int, device) -> Dict:
+    cfg = closest_config(s)
+    model = build_model(cfg, torch.bfloat16, device, seed=0)
+    gen = Generator(model, max_batch=batch, max_seq=prompt + steps + 16)
+    gen.b1 = False
+    ids = torch.randint(0, s["vocab"], (1, prompt), generator=torch.Generator().manual_seed(0)).to(device)
+    t_pre = _timed(lambda: gen.prefill(ids, 0, 0), 3)
+    sp = SamplingParams(max_new_tokens=steps + 8, do_sample=False, repetition_penalty=1.0)
+    gen.start([ids[0].tolist()] * batch, sp)
+    gen.step(3, record_latency=False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    gen.step(steps, record_latency=False)
+    torch.cuda.synchronize()
+    t_dec = (time.perf_counter() - t0) / steps
+    return {"prefill_tok_s": prompt / t_pre, "prefill_ms": t_pre * 1e3, "decode_tok_s": batch / t_dec,
+            "decode_ms_per_step": t_dec * 1e3}
+
+
+def run(sizes: List[str], prompt: int = 4096, batch: int = 4, steps: int = 32, device=None) -> Dict:
+    device = torch.device(device or "cuda:0")
+    res = {}
+    for name in sizes:
+        s = SIZES[name]
+        h = bench_hybrid(s, prompt, batch, steps, device)
+        torch.cuda.empty_cache()
+        c = bench_closest(s, prompt, batch, steps, device)
+        torch.cuda.empty_cache()
+        r2 = lambda d: {k: (round(v, 2) if isinstance(v, float) else v) for k, v in d.items()}
+        res[name] = {"size": s, "nudadra": r2(h), "closest_phi_layout": r2(c),
+                     "prefill_ratio": round(h["prefill_tok_s"] / c["prefill_tok_s"], 3),
+                     "decode_ratio": round(h["decode_tok_s"] / c["decode_tok_s"], 3)}
+    return {"metric": "prefill / decode tokens/s, Nudadra layer-spec model vs the parallel-residual decoder of equal size",
+            "dtype": "bf16", "data": "synthetic (random weights, random prompt)", "prompt_tokens": prompt,
+            "decode_batch": batch, "decode_steps": steps, "sizes": res}

@@ -35,6 +35,10 @@ int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, cons
 int edge_sm_ssd_scan(const void* xbc, int Cx, const void* u, int ld, int dt0, const float* dt_bias, const float* A_log,
                      const float* Dp, float* state, const int* seq_slot, const int* seq_start, const int* seq_len,
                      const int* seq_off, float* y, int n, int Hs, int P, int N, int groups, int f32, hipStream_t st);
+int edge_sm_ssd_chunked(const void* xbc, int Cx, const void* u, int ld, int dt0, const float* dt_bias,
+                        const float* A_log, const float* Dp, float* state, const int* seq_slot, const int* seq_start,
+                        const int* seq_len, const int* seq_off, float* y, float* sloc, float* cdec, int n,
+                        int max_chunks, int Hs, int P, int N, int groups, int f32, hipStream_t st);
 }
 
 namespace {
@@ -252,7 +256,7 @@ at::Tensor sm_conv_silu(const at::Tensor& u, int64_t c0, int64_t C, const at::Te
 at::Tensor sm_ssd_scan(const at::Tensor& xbc, const at::Tensor& u, int64_t dt0, const at::Tensor& dt_bias,
                        const at::Tensor& A_log, const at::Tensor& D, at::Tensor& state, const at::Tensor& seq_slot,
                        const at::Tensor& seq_start, const at::Tensor& seq_len, const at::Tensor& seq_off, int64_t n,
-                       int64_t Hs, int64_t P, int64_t N, int64_t groups) {
+                       int64_t Hs, int64_t P, int64_t N, int64_t groups, int64_t chunks, int64_t max_chunks) {
   const int ld = row_ld(u, "u");
   chk_f32(dt_bias, "dt_bias");
   chk_f32(A_log, "A_log");
@@ -270,6 +274,19 @@ at::Tensor sm_ssd_scan(const at::Tensor& xbc, const at::Tensor& u, int64_t dt0, 
               "sequence metadata: [n]");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(xbc.device());
   auto y = at::empty({xbc.size(0), Hs * P}, xbc.options().dtype(at::kFloat));
+  if (chunks > 0) {
+    // long portions: the chunked form (chunks = sum of ceil(len / 64) over the step's sequences)
+    TORCH_CHECK(chunks * 64 >= xbc.size(0) && max_chunks <= chunks, "chunk counts do not cover the step");
+    auto sloc = at::empty({chunks, Hs, N, P}, y.options());
+    auto cdec = at::empty({chunks, Hs}, y.options());
+    check(edge_sm_ssd_chunked(xbc.data_ptr(), (int)xbc.size(1), u.data_ptr(), ld, (int)dt0, dt_bias.data_ptr<float>(),
+                              A_log.data_ptr<float>(), D.data_ptr<float>(), state.data_ptr<float>(),
+                              seq_slot.data_ptr<int>(), seq_start.data_ptr<int>(), seq_len.data_ptr<int>(),
+                              seq_off.data_ptr<int>(), y.data_ptr<float>(), sloc.data_ptr<float>(), cdec.data_ptr<float>(),
+                              (int)n, (int)max_chunks, (int)Hs, (int)P, (int)N, (int)groups, f32(xbc), stream()),
+          "sm_ssd_chunked");
+    return y;
+  }
   check(edge_sm_ssd_scan(xbc.data_ptr(), (int)xbc.size(1), u.data_ptr(), ld, (int)dt0, dt_bias.data_ptr<float>(),
                          A_log.data_ptr<float>(), D.data_ptr<float>(), state.data_ptr<float>(), seq_slot.data_ptr<int>(),
                          seq_start.data_ptr<int>(), seq_len.data_ptr<int>(), seq_off.data_ptr<int>(), y.data_ptr<float>(),

@@ -422,6 +422,201 @@ __global__ void __launch_bounds__(64) ssd_kernel(const T* __restrict__ xbc, int 
   }
 }
 
+
+// ---------------------------------------------------------------------------------- chunked recurrence
+// The same recurrence for long portions, in chunks of CL tokens (state-space duality): with
+// la_t = -exp(A_log) * (dt_1 + .. + dt_t) inside a chunk,
+//   S_t = e^{la_t} S_in + sum_{s<=t} e^{la_t - la_s} dt_s B_s x_s^T
+//   y_t = e^{la_t} C_t^T S_in + sum_{s<=t} (C_t . B_s) e^{la_t - la_s} dt_s x_s + D x_t
+// (1) every chunk's own contribution to its end state, all chunks in parallel; (2) the states at
+// the chunk borders, one short pass per sequence; (3) every chunk's outputs, all chunks in parallel.
+// All fp32 FMAs; every exponent is <= 0.
+constexpr int CL = 64;
+
+__device__ __forceinline__ int chunk_base(const int* __restrict__ seq_len, int s) {
+  int b = 0;
+  for (int i = 0; i < s; ++i) b += (seq_len[i] + CL - 1) / CL;
+  return b;
+}
+
+// step sizes and inclusive log-decay of one chunk into LDS (first wave; tc <= 64 tokens)
+template <typename T>
+__device__ __forceinline__ void chunk_steps(const T* __restrict__ u, int ld, int dt0, int h, float bias, float a,
+                                            size_t row0, int tc, float* dt_s, float* la_s) {
+  if (threadIdx.x < 64) {
+    const int t = threadIdx.x;
+    float dt = 0.f;
+    if (t < tc) {
+      const float raw = ldf<T>(u + (row0 + t) * ld + dt0 + h) + bias;
+      dt = raw > 20.f ? raw : log1pf(expf(raw));
+    }
+    float v = -a * dt;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const float w = __shfl_up(v, o, 64);
+      if (t >= o) v += w;
+    }
+    dt_s[t] = dt;
+    la_s[t] = v;
+  }
+}
+
+// (1) Sloc[n][p] = sum_s e^{la_end - la_s} dt_s B_s[n] x_s[p] for one 64 x 64 tile of (n, p)
+template <typename T>
+__global__ void __launch_bounds__(NT) ssd_chunk_state_kernel(
+    const T* __restrict__ xbc, int Cx, const T* __restrict__ u, int ld, int dt0, const float* __restrict__ dt_bias,
+    const float* __restrict__ A_log, const int* __restrict__ seq_len, const int* __restrict__ seq_off,
+    float* __restrict__ sloc, float* __restrict__ cdec, int Hs, int P, int N, int groups, int ntn, int ntp) {
+  __shared__ float dt_s[CL], la_s[CL], B_s[CL][CL + 1], X_s[CL][CL + 1];
+  const int tile = blockIdx.x % (ntn * ntp), c = blockIdx.x / (ntn * ntp), s = blockIdx.y, h = blockIdx.z;
+  const int len = seq_len[s];
+  if (c * CL >= len) return;
+  const int tc = min(CL, len - c * CL), n0 = (tile / ntp) * CL, p0 = (tile % ntp) * CL;
+  const size_t row0 = (size_t)seq_off[s] + (size_t)c * CL;
+  const int g = h / (Hs / groups), inner = Hs * P, tid = threadIdx.x;
+  chunk_steps<T>(u, ld, dt0, h, dt_bias[h], expf(A_log[h]), row0, tc, dt_s, la_s);
+  __syncthreads();
+  const float la_end = la_s[tc - 1];
+  for (int e = tid; e < CL * CL; e += NT) {
+    const int t = e / CL, j = e % CL;
+    const bool ok = t < tc;
+    B_s[t][j] = ok && n0 + j < N ? ldf<T>(xbc + (row0 + t) * Cx + inner + g * N + n0 + j) : 0.f;
+    X_s[t][j] = ok && p0 + j < P ? ldf<T>(xbc + (row0 + t) * Cx + h * P + p0 + j) * (expf(la_end - la_s[t]) * dt_s[t]) : 0.f;
+  }
+  __syncthreads();
+  const int ty = tid / 16, tx = tid % 16;
+  float acc[4][4] = {};
+  for (int t = 0; t < tc; ++t) {
+    float b[4], x[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { b[i] = B_s[t][ty * 4 + i]; x[i] = X_s[t][tx * 4 + i]; }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] += b[i] * x[j];
+  }
+  const size_t cb = (size_t)chunk_base(seq_len, s) + c;
+  float* dst = sloc + (cb * Hs + h) * (size_t)N * P;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + ty * 4 + i, p = p0 + tx * 4 + j;
+      if (n < N && p < P) dst[(size_t)n * P + p] = acc[i][j];
+    }
+  if (tile == 0 && tid == 0) cdec[cb * Hs + h] = expf(la_end);
+}
+
+// (2) the state entering every chunk (written over that chunk's own contribution) and the final state
+__global__ void __launch_bounds__(NT) ssd_chunk_scan_kernel(float* __restrict__ sloc, const float* __restrict__ cdec,
+                                                            float* __restrict__ state,
+                                                            const int* __restrict__ seq_slot,
+                                                            const int* __restrict__ seq_start,
+                                                            const int* __restrict__ seq_len, int Hs, int NP) {
+  const int s = blockIdx.x, h = blockIdx.y, e = blockIdx.z * NT + threadIdx.x;
+  if (e >= NP) return;
+  const int nc = (seq_len[s] + CL - 1) / CL;
+  const size_t cb = chunk_base(seq_len, s);
+  float* st = state + ((size_t)seq_slot[s] * Hs + h) * NP + e;
+  float S = seq_start[s] > 0 ? *st : 0.f;
+  for (int c = 0; c < nc; ++c) {
+    float* q = sloc + ((cb + c) * Hs + h) * (size_t)NP + e;
+    const float own = *q;
+    *q = S;
+    S = cdec[(cb + c) * Hs + h] * S + own;
+  }
+  *st = S;
+}
+
+// (3) y for one chunk and 64 value columns
+template <typename T>
+__global__ void __launch_bounds__(NT) ssd_chunk_out_kernel(
+    const T* __restrict__ xbc, int Cx, const T* __restrict__ u, int ld, int dt0, const float* __restrict__ dt_bias,
+    const float* __restrict__ A_log, const float* __restrict__ Dp, const int* __restrict__ seq_len,
+    const int* __restrict__ seq_off, const float* __restrict__ sin_, float* __restrict__ y, int Hs, int P, int N,
+    int groups, int ntp) {
+  constexpr int NK = 32;
+  __shared__ float dt_s[CL], la_s[CL], M_s[CL][CL + 1];
+  __shared__ float buf[2 * CL * (NK + 1) + NK * CL];          // C tile | B tile | S_in tile; later the x tile
+  float(*C_s)[NK + 1] = reinterpret_cast<float(*)[NK + 1]>(buf);
+  float(*B_s)[NK + 1] = reinterpret_cast<float(*)[NK + 1]>(buf + CL * (NK + 1));
+  float(*S_s)[CL] = reinterpret_cast<float(*)[CL]>(buf + 2 * CL * (NK + 1));
+  float(*X_s)[CL + 1] = reinterpret_cast<float(*)[CL + 1]>(buf);
+  static_assert(CL * (CL + 1) <= 2 * CL * (NK + 1) + NK * CL, "x tile fits the staging buffer");
+  const int pt = blockIdx.x % ntp, c = blockIdx.x / ntp, s = blockIdx.y, h = blockIdx.z;
+  const int len = seq_len[s];
+  if (c * CL >= len) return;
+  const int tc = min(CL, len - c * CL), p0 = pt * CL;
+  const size_t row0 = (size_t)seq_off[s] + (size_t)c * CL;
+  const int g = h / (Hs / groups), inner = Hs * P, tid = threadIdx.x, ty = tid / 16, tx = tid % 16;
+  chunk_steps<T>(u, ld, dt0, h, dt_bias[h], expf(A_log[h]), row0, tc, dt_s, la_s);
+  const float* sin_c = sin_ + (((size_t)chunk_base(seq_len, s) + c) * Hs + h) * (size_t)N * P;
+  float accm[4][4] = {}, acci[4][4] = {};
+  for (int n0 = 0; n0 < N; n0 += NK) {
+    __syncthreads();
+    for (int e = tid; e < CL * NK; e += NT) {
+      const int t = e / NK, j = e % NK;
+      const bool ok = t < tc && n0 + j < N;
+      const T* row = xbc + (row0 + t) * Cx + inner + g * N + n0 + j;
+      B_s[t][j] = ok ? ldf<T>(row) : 0.f;
+      C_s[t][j] = ok ? ldf<T>(row + groups * N) : 0.f;
+    }
+    for (int e = tid; e < NK * CL; e += NT) {
+      const int j = e / CL, p = e % CL;
+      S_s[j][p] = n0 + j < N && p0 + p < P ? sin_c[(size_t)(n0 + j) * P + p0 + p] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int k = 0; k < NK; ++k) {
+      float cv[4], bv[4], sv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { cv[i] = C_s[ty * 4 + i][k]; bv[i] = B_s[tx * 4 + i][k]; sv[i] = S_s[k][tx * 4 + i]; }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { accm[i][j] += cv[i] * bv[j]; acci[i][j] += cv[i] * sv[j]; }
+    }
+  }
+  // M[t][s'] = (C_t . B_s') e^{la_t - la_s'} dt_s' for s' <= t
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = ty * 4 + i, sp = tx * 4 + j;
+      M_s[t][sp] = (sp <= t && t < tc) ? accm[i][j] * expf(la_s[t] - la_s[sp]) * dt_s[sp] : 0.f;
+    }
+  __syncthreads();                                            // every wave is done with the C / B / S_in tiles
+  for (int e = tid; e < CL * CL; e += NT) {
+    const int t = e / CL, p = e % CL;
+    X_s[t][p] = t < tc && p0 + p < P ? ldf<T>(xbc + (row0 + t) * Cx + h * P + p0 + p) : 0.f;
+  }
+  __syncthreads();
+  float out[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float el = expf(la_s[ty * 4 + i]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[i][j] = el * acci[i][j];
+  }
+  for (int sp = 0; sp < tc; ++sp) {
+    float mv[4], xv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { mv[i] = M_s[ty * 4 + i][sp]; xv[i] = X_s[sp][tx * 4 + i]; }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) out[i][j] += mv[i] * xv[j];
+  }
+  const float Dh = Dp[h];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int t = ty * 4 + i, p = p0 + tx * 4 + j;
+      if (t < tc && p < P) y[(row0 + t) * inner + h * P + p] = out[i][j] + Dh * X_s[t][tx * 4 + j];
+    }
+}
+
 }  // namespace
 
 #define SM_T(f32, ...)                                  \
@@ -555,6 +750,26 @@ int edge_sm_ssd_scan(const void* xbc, int Cx, const void* u, int ld, int dt0, co
   else if (N <= 128) SM_SSD(128);
   else SM_SSD(256);
 #undef SM_SSD
+  return (int)hipGetLastError();
+}
+
+// chunked form for long portions: scratch sloc [chunks, Hs, N, P] and cdec [chunks, Hs] (fp32);
+// chunks = sum over sequences of ceil(len / 64), max_chunks = the largest of them
+int edge_sm_ssd_chunked(const void* xbc, int Cx, const void* u, int ld, int dt0, const float* dt_bias,
+                        const float* A_log, const float* Dp, float* state, const int* seq_slot, const int* seq_start,
+                        const int* seq_len, const int* seq_off, float* y, float* sloc, float* cdec, int n,
+                        int max_chunks, int Hs, int P, int N, int groups, int f32, hipStream_t st) {
+  if (n == 0 || max_chunks <= 0) return 0;
+  if (groups <= 0 || Hs % groups) return -2;
+  const int ntn = (N + CL - 1) / CL, ntp = (P + CL - 1) / CL;
+  SM_T(f32, hipLaunchKernelGGL(ssd_chunk_state_kernel<T>, dim3(max_chunks * ntn * ntp, n, Hs), dim3(NT), 0, st,
+                               (const T*)xbc, Cx, (const T*)u, ld, dt0, dt_bias, A_log, seq_len, seq_off, sloc, cdec, Hs,
+                               P, N, groups, ntn, ntp));
+  hipLaunchKernelGGL(ssd_chunk_scan_kernel, dim3(n, Hs, (N * P + NT - 1) / NT), dim3(NT), 0, st, sloc, cdec, state,
+                     seq_slot, seq_start, seq_len, Hs, N * P);
+  SM_T(f32, hipLaunchKernelGGL(ssd_chunk_out_kernel<T>, dim3(max_chunks * ntp, n, Hs), dim3(NT), 0, st, (const T*)xbc,
+                               Cx, (const T*)u, ld, dt0, dt_bias, A_log, Dp, seq_len, seq_off, sloc, y, Hs, P, N, groups,
+                               ntp));
   return (int)hipGetLastError();
 }
 

@@ -304,6 +304,9 @@ def conv_silu(u: torch.Tensor, c0: int, C: int, weight: torch.Tensor, bias: torc
     return out
 
 
+SSD_CHUNK_MIN = int(__import__("os").environ.get("EDGELLM_SSD_CHUNK_MIN", "32"))
+
+
 def ssd_scan(xbc: torch.Tensor, u: torch.Tensor, dt0: int, dt_bias, A_log, D, state: torch.Tensor,
              meta: RaggedMeta, heads: int, vdim: int, N: int, groups: int) -> torch.Tensor:
     """The state-space recurrence, token by token in fp32.  xbc [T, x | B | C] (after conv + silu),
@@ -312,8 +315,15 @@ def ssd_scan(xbc: torch.Tensor, u: torch.Tensor, dt0: int, dt_bias, A_log, D, st
     read (zero for a portion starting at 0) and left at the portion's end.  Returns y fp32 [T, inner]."""
     inner = heads * vdim
     if _gpu(xbc):
+        # portions of SSD_CHUNK_MIN tokens or more: the chunked (state-space duality) kernels, parallel
+        # over chunks of 64 tokens; shorter steps (decode): one wave per (sequence, head) token by token
+        chunks = max_chunks = 0
+        if meta.max_len >= SSD_CHUNK_MIN:
+            per = [(h[2] + 63) // 64 for h in meta.host]
+            chunks, max_chunks = sum(per), max(per)
         return _ext().sm_ssd_scan(xbc, u, int(dt0), dt_bias, A_log, D, state, meta.seq_slot, meta.seq_start,
-                                  meta.seq_len, meta.seq_off, int(meta.n), int(heads), int(vdim), int(N), int(groups))
+                                  meta.seq_len, meta.seq_off, int(meta.n), int(heads), int(vdim), int(N), int(groups),
+                                  int(chunks), int(max_chunks))
     T = xbc.shape[0]
     y = torch.empty(T, inner, dtype=torch.float32, device=xbc.device)
     a = torch.exp(A_log.float())

@@ -200,13 +200,17 @@ def test_attention_op_portions_and_a_far_key(dev, window, pool, H, G, D, Dv, pag
 
 
 @pytest.mark.parametrize("dev", DEVS)
-@pytest.mark.parametrize("Hs,P,N,groups,taps", [(2, 4, 3, 1, 4), (4, 8, 16, 2, 2), (3, 5, 20, 3, 5), (1, 70, 33, 1, 3)])
-def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps):
-    """Convolution tail and state matrix carried over portions of 1..5 tokens, two sequences
-    interleaved in the same steps, against one pass of the oracle over each whole sequence."""
+@pytest.mark.parametrize("Hs,P,N,groups,taps,sizes", [
+    (2, 4, 3, 1, 4, (1, 2, 3, 4, 5)), (4, 8, 16, 2, 2, (1, 2, 3, 4, 5)), (3, 5, 20, 3, 5, (1, 2, 3, 4, 5)),
+    (1, 70, 33, 1, 3, (1, 2, 3, 4, 5)), (2, 70, 67, 2, 4, (64, 1, 33, 65, 2, 130)), (3, 16, 8, 1, 3, (40, 100, 7))])
+def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps, sizes):
+    """Convolution tail and state matrix carried over portions of ``sizes`` tokens (short ones step
+    token by token, long ones take the chunked form; chunk borders inside and at the end of a
+    portion), two sequences interleaved in the same steps, against one pass of the oracle over each
+    whole sequence."""
     torch.manual_seed(2)
     inner, C = Hs * P, Hs * P + 2 * groups * N
-    Ts = {0: 23, 2: 17}
+    Ts = {0: 23, 2: 17} if max(sizes) < 10 else {0: 300, 2: 171}
     u = {s: torch.randn(T, 2 * inner + 2 * groups * N + Hs, dtype=torch.float64) for s, T in Ts.items()}
     cw, cb = torch.randn(C, taps, dtype=torch.float64) * 0.5, torch.randn(C, dtype=torch.float64) * 0.2
     dtb, A_log, Dp = torch.randn(Hs, dtype=torch.float64), torch.rand(Hs, dtype=torch.float64) - 0.5, torch.randn(Hs, dtype=torch.float64)
@@ -221,9 +225,11 @@ def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps):
     f = lambda t: t.float().to(dev)
     conv = torch.full((3, max(taps - 1, 1), C), 7.0, device=dev)       # stale rows of an earlier tenant
     ssm = torch.full((3, Hs, N, P), -3.0, device=dev)
-    at, got, n = {s: 0 for s in Ts}, {s: [] for s in Ts}, 1
+    at, got, k = {s: 0 for s in Ts}, {s: [] for s in Ts}, 0
     pt = torch.zeros(3, 4, dtype=torch.int32, device=dev)
     while any(at[s] < Ts[s] for s in Ts):
+        n = sizes[k % len(sizes)]
+        k += 1
         seqs = [(s, at[s], min(n + (s == 2), Ts[s] - at[s])) for s in Ts if at[s] < Ts[s]]
         meta = seqmix.RaggedMeta.build(seqs, pt, 64, dev)
         uu = f(torch.cat([u[s][a:a + m] for s, a, m in seqs]))
@@ -235,7 +241,6 @@ def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps):
             got[s].append(o[off:off + m])
             off += m
             at[s] += m
-        n = n % 5 + 1
     for s in Ts:
         assert torch.allclose(torch.cat(got[s]), want[s], atol=3e-5, rtol=1e-4), s
 
