@@ -29,14 +29,71 @@ from .generate import GenerationResult, SamplingParams
 from .paged import PagedCache
 
 
+class _DecodeGraph:
+    """A captured decode step for ``n`` sequences (one token each): static token / metadata buffers
+    filled from pinned host rows before every replay; the first call runs eagerly (lazy weight packs
+    and rotary tables are built outside any capture)."""
+    RING = 8
+
+    def __init__(self, eng: "RaggedEngine", n: int):
+        dev = eng.device
+        self.eng, self.n = eng, n
+        self.buf = torch.zeros(6 * n, dtype=torch.int32, device=dev)
+        self.ids = torch.zeros(n, dtype=torch.long, device=dev)
+        self.host = [(torch.zeros(6 * n, dtype=torch.int32).pin_memory(), torch.zeros(n, dtype=torch.long).pin_memory(),
+                      torch.cuda.Event()) for _ in range(self.RING)]
+        self.turn = 0
+        b = self.buf
+        cap = eng.cache.num_pages * eng.page
+        self.meta = RaggedMeta(n, n, b[0:n], b[n:2 * n], b[2 * n:3 * n], b[3 * n:4 * n], b[4 * n:5 * n], b[5 * n:6 * n],
+                               eng.cache.page_table, eng.page, [(0, 1, 1, i) for i in range(n)], 1, cap)
+        self.rows = torch.arange(n, dtype=torch.long, device=dev)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.out: Optional[torch.Tensor] = None
+        self.warm = False
+
+    def run(self, seqs, ids) -> torch.Tensor:
+        n = self.n
+        hb, hi, ev = self.host[self.turn]
+        self.turn = (self.turn + 1) % self.RING
+        ev.synchronize()                           # the copy that last read this pinned row is done
+        flat = [s[0] for s in seqs] + [s[1] for s in seqs] + [1] * n + list(range(n)) + list(range(n)) + \
+            [s[1] for s in seqs]
+        hb.copy_(torch.tensor(flat, dtype=torch.int32))
+        hi.copy_(torch.tensor(ids, dtype=torch.long))
+        self.buf.copy_(hb, non_blocking=True)
+        self.ids.copy_(hi, non_blocking=True)
+        ev.record()
+        eng = self.eng
+        if not self.warm:
+            self.warm = True
+            return eng.model(self.ids, self.meta, eng.cache, self.rows)
+        if self.graph is None:
+            g = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(g, pool=eng._pool):
+                self.out = eng.model(self.ids, self.meta, eng.cache, self.rows)
+            if eng._pool is None:
+                eng._pool = g.pool()
+            self.graph = g
+        self.graph.replay()
+        return self.out
+
+
 class RaggedEngine:
-    def __init__(self, model, max_tokens: int, slots: int = 4, page: int = 64):
+    def __init__(self, model, max_tokens: int, slots: int = 4, page: int = 64, use_graphs: Optional[bool] = None):
         assert getattr(model, "ragged", False), "RaggedEngine runs layer-spec (ragged-step) models"
         self.model, self.cfg, self.device = model, model.cfg, model.device
         self.page = page
         pages = max(1, (int(max_tokens) + page - 1) // page)
         self.cache = PagedCache(model.run_specs(), pages, slots, page, dtype=model.dtype, device=self.device)
         self.live: Dict[object, int] = {}
+        # decode-only steps (every sequence brings one token) replay a HIP graph per batch size
+        self.use_graphs = (self.device.type == "cuda" and ops.gpu_path(model.embed)) if use_graphs is None \
+            else bool(use_graphs)
+        self._graphs: Dict[int, _DecodeGraph] = {}
+        self._pool = None
+        self.graphs_used = False
 
     # ------------------------------------------------------------------ requests
     def open(self, rid) -> int:
@@ -72,6 +129,16 @@ class RaggedEngine:
             off += len(toks)
         if not seqs:
             return torch.empty(0, self.cfg.vocab_size, dtype=torch.float32, device=self.device)
+        if self.use_graphs and taps is None and len(ids) == len(seqs):
+            dg = self._graphs.get(len(seqs))
+            if dg is None:
+                dg = self._graphs[len(seqs)] = _DecodeGraph(self, len(seqs))
+            with trace_range(f"ragged.decode.n{len(seqs)}"):
+                out = dg.run(seqs, ids)
+            self.graphs_used = self.graphs_used or dg.graph is not None
+            if rows == list(range(len(seqs))):
+                return out.clone()
+            return out.index_select(0, torch.tensor(rows, dtype=torch.long, device=self.device))
         meta = RaggedMeta.build(seqs, self.cache.page_table, self.page, self.device)
         ids_t = torch.tensor(ids, dtype=torch.long, device=self.device)
         rows_t = torch.tensor(rows, dtype=torch.long, device=self.device)

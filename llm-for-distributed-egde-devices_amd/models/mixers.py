@@ -20,6 +20,10 @@ from .configs import SSDSpec, WindowAttnSpec
 from .layers import Linear
 
 
+_ROPE_TABLES: dict = {}
+_ROPE_RETIRED: list = []
+
+
 class WindowPoolAttention(nn.Module):
     """Grouped-query softmax attention whose query at position i sees the last ``window`` tokens
     and one mean key / value per block of ``pool`` tokens lying wholly before the window
@@ -33,12 +37,23 @@ class WindowPoolAttention(nn.Module):
         self._rope = None
 
     def rope(self, n: int, device) -> Optional[torch.Tensor]:
+        """cos / sin rows for positions [0, n): one table per (rotation constants, device), shared by
+        every layer that rotates alike, grown by doubling."""
         s = self.spec
         if not s.rot_dims:
             return None
         if self._rope is None or self._rope.shape[0] < n or self._rope.device != torch.device(device):
-            from .. import ops
-            self._rope = ops.rope_tables(s.rot_dims, max(n, 2048), s.rot_base, s.rot_scaling, device=device)
+            key = (s.rot_dims, s.rot_base, tuple(sorted((s.rot_scaling or {}).items())), str(torch.device(device)))
+            tab = _ROPE_TABLES.get(key)
+            if tab is None or tab.shape[0] < n:
+                from .. import ops
+                rows = 2048
+                while rows < n:
+                    rows *= 2
+                if tab is not None:
+                    _ROPE_RETIRED.append(tab)           # a captured graph may still read the smaller table
+                tab = _ROPE_TABLES[key] = ops.rope_tables(s.rot_dims, rows, s.rot_base, s.rot_scaling, device=device)
+            self._rope = tab
         return self._rope
 
     def forward(self, u: torch.Tensor, c0: int, meta: seqmix.RaggedMeta, run) -> torch.Tensor:

@@ -28,6 +28,11 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
                       int window, int pool, int f32, hipStream_t st);
+int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp,
+                           const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
+                           const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
+                           int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
+                           int pool, hipStream_t st);
 int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
                       const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
                       const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
@@ -197,7 +202,9 @@ void sm_pool_blocks(const at::Tensor& kp, const at::Tensor& vp, at::Tensor& kb, 
 at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& gate, const at::Tensor& kp,
                         const at::Tensor& vp, const std::optional<at::Tensor>& kb, const std::optional<at::Tensor>& vb,
                         const at::Tensor& tok_seq, const at::Tensor& tok_pos, const at::Tensor& seq_slot,
-                        const at::Tensor& ptab, double scale, int64_t window, int64_t pool, int64_t max_keys) {
+                        const at::Tensor& ptab, double scale, int64_t window, int64_t pool, int64_t max_keys,
+                        const std::optional<at::Tensor>& seq_start, const std::optional<at::Tensor>& seq_len,
+                        const std::optional<at::Tensor>& seq_off, int64_t n, int64_t qtiles) {
   chk_i32(tok_seq, "tok_seq");
   chk_i32(tok_pos, "tok_pos");
   chk_i32(seq_slot, "seq_slot");
@@ -222,6 +229,26 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
   }
   c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
   auto out = at::empty({T, H * Dv}, q.options());
+  if (qtiles > 0 && q.scalar_type() == at::kBFloat16) {
+    // prompt portions in bf16 (qtiles = sum of ceil(len / 64)): the MFMA kernel when it takes the head sizes
+    TORCH_CHECK(seq_start && seq_len && seq_off, "sequence metadata missing");
+    chk_i32(*seq_start, "seq_start");
+    chk_i32(*seq_len, "seq_len");
+    chk_i32(*seq_off, "seq_off");
+    TORCH_CHECK(seq_start->numel() >= n && seq_len->numel() >= n && seq_off->numel() >= n && seq_slot.numel() >= n &&
+                    qtiles * 64 >= T, "sequence metadata: [n]");
+    const int rc = edge_sm_attention_mfma(q.data_ptr(), gate ? gate->data_ptr() : nullptr, gate_ld, kp.data_ptr(),
+                                          vp.data_ptr(), PB ? kb->data_ptr<float>() : nullptr,
+                                          PB ? vb->data_ptr<float>() : nullptr, seq_slot.data_ptr<int>(),
+                                          seq_start->data_ptr<int>(), seq_len->data_ptr<int>(), seq_off->data_ptr<int>(),
+                                          ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)n, (int)qtiles,
+                                          (int)H, (int)G, (int)D, (int)Dv, (int)page, PB, (float)scale, (int)window,
+                                          PB ? (int)pool : 0, stream());
+    if (rc != 1) {
+      check(rc, "sm_attention_mfma");
+      return out;
+    }
+  }
   check(edge_sm_attention(q.data_ptr(), gate ? gate->data_ptr() : nullptr, gate_ld, kp.data_ptr(), vp.data_ptr(),
                           PB ? kb->data_ptr<float>() : nullptr, PB ? vb->data_ptr<float>() : nullptr,
                           tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),

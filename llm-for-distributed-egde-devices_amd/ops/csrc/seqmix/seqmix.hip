@@ -175,7 +175,16 @@ __global__ void __launch_bounds__(NT) pool_kernel(const T* __restrict__ kp, cons
 // pooled blocks (fp32 rows): one softmax over both.
 constexpr int KC = 256;
 
-template <typename KT, int RMAX, int DVL>
+template <typename KT> __device__ __forceinline__ void load8(const KT* p, float* f);
+template <> __device__ __forceinline__ void load8<float>(const float* p, float* f) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float* f) {
+  unpack8(*reinterpret_cast<const uint4*>(p), f);
+}
+
+template <typename KT, int RMAX, int DVL, bool VEC>
 __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const KT* __restrict__ vbase, int cnt, int g,
                                            int G, int D, int Dv, int R, const float* q_s, float* s_s, int* row_s,
                                            float* m_s, float* l_s, float* a_s, int rowidx, float (&acc)[RMAX][DVL]) {
@@ -187,10 +196,21 @@ __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const K
     for (int r = 0; r < RMAX; ++r) a[r] = 0.f;
     if (tid < cnt) {
       const KT* kr = kbase + ((size_t)rowidx * G + g) * D;
-      for (int d = 0; d < D; ++d) {
-        const float kv = ldf<KT>(kr + d);
+      if constexpr (VEC) {                                  // rows are 16-byte aligned: D % 8 == 0
+        for (int d = 0; d < D; d += 8) {
+          float kv[8];
+          load8<KT>(kr + d, kv);
 #pragma unroll
-        for (int r = 0; r < RMAX; ++r) a[r] += q_s[r * D + d] * kv;
+          for (int e = 0; e < 8; ++e)
+#pragma unroll
+            for (int r = 0; r < RMAX; ++r) a[r] += q_s[r * D + d + e] * kv[e];
+        }
+      } else {
+        for (int d = 0; d < D; ++d) {
+          const float kv = ldf<KT>(kr + d);
+#pragma unroll
+          for (int r = 0; r < RMAX; ++r) a[r] += q_s[r * D + d] * kv;
+        }
       }
     }
 #pragma unroll
@@ -228,32 +248,44 @@ __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const K
 #pragma unroll
     for (int dl = 0; dl < DVL; ++dl) acc[r][dl] *= al;
   }
+  // eight rows' loads are issued before their products (the walk is latency-bound otherwise)
   const int j1 = min(cnt, 64 * (wave + 1));
-  for (int j = 64 * wave; j < j1; ++j) {
-    const KT* vr = vbase + ((size_t)row_s[j] * G + g) * Dv;
-    float vv[DVL];
+  constexpr int UN = 8;
+  for (int j = 64 * wave; j < j1; j += UN) {
+    float vv[UN][DVL];
 #pragma unroll
-    for (int dl = 0; dl < DVL; ++dl) vv[dl] = lane + 64 * dl < Dv ? ldf<KT>(vr + lane + 64 * dl) : 0.f;
+    for (int k = 0; k < UN; ++k) {
+      const KT* vr = vbase + ((size_t)row_s[min(j + k, j1 - 1)] * G + g) * Dv;
 #pragma unroll
-    for (int r = 0; r < RMAX; ++r) {
-      const float p = s_s[r * KC + j];
+      for (int dl = 0; dl < DVL; ++dl) vv[k][dl] = lane + 64 * dl < Dv ? ldf<KT>(vr + lane + 64 * dl) : 0.f;
+    }
 #pragma unroll
-      for (int dl = 0; dl < DVL; ++dl) acc[r][dl] += p * vv[dl];
+    for (int k = 0; k < UN; ++k) {
+      if (j + k < j1) {
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r) {
+          const float p = s_s[r * KC + j + k];
+#pragma unroll
+          for (int dl = 0; dl < DVL; ++dl) acc[r][dl] += p * vv[k][dl];
+        }
+      }
     }
   }
   __syncthreads();
 }
 
-template <typename T, int RMAX, int DVL>
+template <typename T, int RMAX, int DVL, bool VEC>
 __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const T* __restrict__ gate, int gate_ld,
                                                   const T* __restrict__ kp, const T* __restrict__ vp,
                                                   const float* __restrict__ kb, const float* __restrict__ vb,
                                                   const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                                   const int* __restrict__ seq_slot, const int* __restrict__ ptab,
                                                   int ptab_ld, T* __restrict__ out, int H, int G, int D, int Dv,
-                                                  int page, int PB, float scale, int window, int pool) {
+                                                  int page, int PB, float scale, int window, int pool, int nsp) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  const int t = blockIdx.x, g = blockIdx.y, R = H / G;
+  // more than RMAX query heads per kv head: nsp workgroups share the kv head, RMAX heads each
+  const int t = blockIdx.x, g = blockIdx.y / nsp, r0 = (blockIdx.y % nsp) * RMAX;
+  const int R = min(RMAX, H / G - r0), hq0 = g * (H / G) + r0;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   float* q_s = smem;                         // [RMAX][D]
   float* s_s = q_s + RMAX * D;               // [RMAX][KC]
@@ -266,7 +298,7 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
   const int* pt = ptab + (size_t)seq_slot[tok_seq[t]] * ptab_ld;
   for (int e = tid; e < RMAX * D; e += NT) {
     const int r = e / D, d = e % D;
-    q_s[e] = r < R ? ldf<T>(q + ((size_t)t * H + g * R + r) * D + d) * scale : 0.f;
+    q_s[e] = r < R ? ldf<T>(q + ((size_t)t * H + hq0 + r) * D + d) * scale : 0.f;
   }
   for (int e = tid; e < RMAX * Dv; e += NT) red[e] = 0.f;
   if (tid < RMAX) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; }
@@ -282,12 +314,12 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
   for (int c0 = 0; c0 < nt; c0 += KC) {
     const int j = jlo + c0 + tid;
     const int rowidx = c0 + tid < nt ? pt[j / page] * page + j % page : 0;
-    attn_chunk<T, RMAX, DVL>(kp, vp, min(KC, nt - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
+    attn_chunk<T, RMAX, DVL, VEC>(kp, vp, min(KC, nt - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
   }
   for (int c0 = 0; c0 < nb; c0 += KC) {
     const int p0 = (c0 + tid) * pool;
     const int rowidx = c0 + tid < nb ? pt[p0 / page] * PB + (p0 % page) / pool : 0;
-    attn_chunk<float, RMAX, DVL>(kb, vb, min(KC, nb - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
+    attn_chunk<float, RMAX, DVL, VEC>(kb, vb, min(KC, nb - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
   }
   // sum the four waves' partial outputs, normalise, gate
   for (int w = 0; w < NT / 64; ++w) {
@@ -301,10 +333,176 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
     __syncthreads();
   }
   for (int e = tid; e < R * Dv; e += NT) {
-    const int r = e / Dv, h = g * R + r;
+    const int r = e / Dv, h = hq0 + r;
     float o = red[e] / l_s[r];
     if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + h));
     stf<T>(out + ((size_t)t * H + h) * Dv + e % Dv, o);
+  }
+}
+
+// ---------------------------------------------------------------------------------- attention, bf16 MFMA
+// Prompt portions in bf16: 64 query rows of one (sequence, head) per workgroup, 16 per wave, on
+// v_mfma_f32_16x16x32_bf16.  A key tile is one page of the sequence (64 tokens, rows G * D apart) or
+// 64 pooled blocks (fp32 rows rounded to bf16 while staging); per tile S = Q K^T from a padded-row
+// LDS image of K, the mask (window / block-complete rule) and the online softmax in fp32 in the
+// log2 domain, P to per-wave LDS as bf16, O += P V with V fragments read transposed from the
+// row-major V tile.  Tiles wholly outside a workgroup's window are never visited.
+constexpr int MQ = 64, MK = 64;
+
+template <int DK, int DV>
+__global__ void __launch_bounds__(NT) attn_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ gate, int gate_ld, const bf16_t* __restrict__ kp,
+    const bf16_t* __restrict__ vp, const float* __restrict__ kb, const float* __restrict__ vb,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_len,
+    const int* __restrict__ seq_off, const int* __restrict__ ptab, int ptab_ld, bf16_t* __restrict__ out, int n, int H,
+    int G, int PB, float scale_log2, int window, int pool) {
+  constexpr int D = 32 * DK, Dv = 16 * DV;
+  constexpr int KS = D * 2 + 16, VS = Dv * 2 + 16, PS = MK * 2 + 16;      // LDS row strides in bytes
+  __shared__ __attribute__((aligned(16))) char k_lds[MK * KS];
+  __shared__ __attribute__((aligned(16))) char v_lds[MK * VS];
+  __shared__ __attribute__((aligned(16))) char p_all[4 * 16 * PS];
+  typedef __attribute__((address_space(3))) v4s lds_v4s;
+  int qt = blockIdx.x, s = 0;
+  for (; s < n; ++s) {
+    const int nq = (seq_len[s] + MQ - 1) / MQ;
+    if (qt < nq) break;
+    qt -= nq;
+  }
+  if (s == n) return;
+  const int h = blockIdx.y, g = h / (H / G);
+  const int start = seq_start[s], len = seq_len[s], off = seq_off[s];
+  const int* pt = ptab + (size_t)seq_slot[s] * ptab_ld;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, c16 = lane & 15;
+  char* p_lds = p_all + wave * 16 * PS;
+  const int wq0 = qt * MQ + wave * 16;                       // this wave's first row inside the portion
+  v8s qf[DK];
+  {
+    const int t = wq0 + c16;
+#pragma unroll
+    for (int kk = 0; kk < DK; ++kk)
+      qf[kk] = t < len ? *reinterpret_cast<const v8s*>(q + ((size_t)(off + t) * H + h) * D + kk * 32 + 8 * g4)
+                       : v8s{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  v4f o[DV];
+#pragma unroll
+  for (int i = 0; i < DV; ++i) o[i] = v4f{0.f, 0.f, 0.f, 0.f};
+  float m_i[4], l_i[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m_i[i] = -INFINITY; l_i[i] = 0.f; }
+  const int imin = start + qt * MQ, imax = start + min(len, qt * MQ + MQ) - 1;
+  const int jlo = window > 0 ? max(0, imin - window + 1) : 0;
+  const int nbmax = (window > 0 && pool > 0 && imax - window + 1 > 0) ? (imax - window + 1) / pool : 0;
+  const int tok_tiles = imax / MK - jlo / MK + 1, ntiles = tok_tiles + (nbmax + MK - 1) / MK;
+
+  for (int tile = 0; tile < ntiles; ++tile) {
+    const bool tok = tile < tok_tiles;
+    const int base = tok ? (jlo / MK + tile) * MK : (tile - tok_tiles) * MK;   // first position / block of the tile
+    __syncthreads();                                         // every wave is done with the previous tile
+    if (tok) {
+      const size_t prow = (size_t)pt[base / MK] * MK;
+      for (int e = tid; e < MK * (D / 8); e += NT) {
+        const int r = e / (D / 8), c = e % (D / 8);
+        *reinterpret_cast<uint4*>(k_lds + r * KS + c * 16) =
+            *reinterpret_cast<const uint4*>(kp + ((prow + r) * G + g) * D + c * 8);
+      }
+      for (int e = tid; e < MK * (Dv / 8); e += NT) {
+        const int r = e / (Dv / 8), c = e % (Dv / 8);
+        *reinterpret_cast<uint4*>(v_lds + r * VS + c * 16) =
+            *reinterpret_cast<const uint4*>(vp + ((prow + r) * G + g) * Dv + c * 8);
+      }
+    } else {
+      for (int e = tid; e < MK * (D / 8 + Dv / 8); e += NT) {
+        const int r = e / (D / 8 + Dv / 8), c = e % (D / 8 + Dv / 8);
+        const int b = base + r;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (b < nbmax) {
+          const int p0 = b * pool;
+          const size_t row = ((size_t)pt[p0 / MK] * PB + (p0 % MK) / pool) * G + g;
+          float f[8];
+          load8<float>(c < D / 8 ? kb + row * D + c * 8 : vb + row * Dv + (c - D / 8) * 8, f);
+          v = pack8(f);
+        }
+        *reinterpret_cast<uint4*>(c < D / 8 ? k_lds + r * KS + c * 16 : v_lds + r * VS + (c - D / 8) * 16) = v;
+      }
+    }
+    __syncthreads();
+    v4f sc[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      sc[nt] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < DK; ++kk) {
+        const v8s kf = *reinterpret_cast<const v8s*>(k_lds + (nt * 16 + c16) * KS + (kk * 32 + 8 * g4) * 2);
+        sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], kf, sc[nt], 0, 0, 0);
+      }
+    }
+    // lane holds S[row = 4 g4 + i][key = 16 nt + c16]
+    float alpha[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int qpos = start + wq0 + 4 * g4 + i;
+      const int seen = (window > 0 && pool > 0 && qpos - window + 1 > 0) ? (qpos - window + 1) / pool : 0;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int key = base + nt * 16 + c16;
+        const bool vis = tok ? (key <= qpos && (window <= 0 || qpos - key < window)) : key < seen;
+        const float v = vis ? sc[nt][i] * scale_log2 : -INFINITY;
+        sc[nt][i] = v;
+        mx = fmaxf(mx, v);
+      }
+#pragma unroll
+      for (int o_ = 1; o_ < 16; o_ <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o_, 64));
+      const float mnew = fmaxf(m_i[i], mx);
+      const float msafe = (mnew == -INFINITY) ? 0.f : mnew;
+      alpha[i] = __builtin_amdgcn_exp2f(m_i[i] - msafe);
+      float rs = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const float p = __builtin_amdgcn_exp2f(sc[nt][i] - msafe);
+        sc[nt][i] = p;
+        rs += p;
+      }
+#pragma unroll
+      for (int o_ = 1; o_ < 16; o_ <<= 1) rs += __shfl_xor(rs, o_, 64);
+      l_i[i] = l_i[i] * alpha[i] + rs;
+      m_i[i] = mnew;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DV; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[dt][i] *= alpha[i];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<bf16_t*>(p_lds + (4 * g4 + i) * PS + (nt * 16 + c16) * 2) = f2bf(sc[nt][i]);
+    __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): this wave's P rows are in LDS
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const v8s pf = *reinterpret_cast<const v8s*>(p_lds + c16 * PS + (ks * 32 + 8 * g4) * 2);
+      const int key0 = ks * 32 + 8 * g4, qq = c16 >> 2, pp = c16 & 3;
+#pragma unroll
+      for (int dt = 0; dt < DV; ++dt) {
+        const char* a0 = v_lds + (key0 + qq) * VS + (dt * 16 + 4 * pp) * 2;
+        const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(a0));
+        const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(a0 + 4 * VS));
+        const v8s vf = v8s{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[dt], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int t = wq0 + 4 * g4 + i;
+    if (t < len) {
+      float inv = l_i[i] > 0.f ? 1.f / l_i[i] : 0.f;
+      if (gate) inv *= sigmoidf_(bf2f(gate[(size_t)(off + t) * gate_ld + h]));
+#pragma unroll
+      for (int dt = 0; dt < DV; ++dt)
+        out[((size_t)(off + t) * H + h) * Dv + dt * 16 + c16] = f2bf(o[dt][i] * inv);
+    }
   }
 }
 
@@ -695,16 +893,23 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
                       int window, int pool, int f32, hipStream_t st) {
   if (rows == 0) return 0;
-  if (G <= 0 || H % G || Dv > 256 || H / G > 16) return -2;
+  if (G <= 0 || H % G || Dv > 256) return -2;
   const int R = H / G;
   const int rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16;
+  const int nsp = (R + rmax - 1) / rmax;
   const size_t lds = sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 3 * rmax) +
                      sizeof(int) * KC;
   if (lds > 64 * 1024) return -3;
-#define SM_ATT(RM, DL)                                                                                              \
-  SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL>), dim3(rows, G), dim3(NT), lds, st, (const T*)q,            \
+  const bool vec = D % 8 == 0;
+#define SM_ATT_V(RM, DL, V)                                                                                         \
+  SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL, V>), dim3(rows, G * nsp), dim3(NT), lds, st, (const T*)q,         \
                                (const T*)gate, gate_ld, (const T*)kp, (const T*)vp, kb, vb, tok_seq, tok_pos,       \
-                               seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool))
+                               seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool, nsp))
+#define SM_ATT(RM, DL)               \
+  do {                               \
+    if (vec) SM_ATT_V(RM, DL, true); \
+    else SM_ATT_V(RM, DL, false);    \
+  } while (0)
 #define SM_ATT_R(DL)                 \
   switch (rmax) {                    \
     case 1: SM_ATT(1, DL); break;    \
@@ -717,6 +922,7 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
   else { SM_ATT_R(4); }
 #undef SM_ATT_R
 #undef SM_ATT
+#undef SM_ATT_V
   return (int)hipGetLastError();
 }
 
@@ -770,6 +976,31 @@ int edge_sm_ssd_chunked(const void* xbc, int Cx, const void* u, int ld, int dt0,
   SM_T(f32, hipLaunchKernelGGL(ssd_chunk_out_kernel<T>, dim3(max_chunks * ntp, n, Hs), dim3(NT), 0, st, (const T*)xbc,
                                Cx, (const T*)u, ld, dt0, dt_bias, A_log, Dp, seq_len, seq_off, sloc, y, Hs, P, N, groups,
                                ntp));
+  return (int)hipGetLastError();
+}
+
+// bf16 prompt portions on the matrix cores; returns 1 when no instantiation takes (D, Dv): the caller
+// then runs the general kernel
+int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp,
+                           const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
+                           const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
+                           int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
+                           int pool, hipStream_t st) {
+  if (page != MK || G <= 0 || H % G) return 1;
+  if (n == 0 || qtiles == 0) return 0;
+  const float sl2 = scale * 1.4426950408889634f;
+#define SM_MF(DK, DV)                                                                                              \
+  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV>), dim3(qtiles, H), dim3(NT), 0, st, (const bf16_t*)q,              \
+                     (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb, seq_slot,         \
+                     seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window, pool)
+  if (D == 64 && Dv == 64) SM_MF(2, 4);
+  else if (D == 96 && Dv == 96) SM_MF(3, 6);
+  else if (D == 128 && Dv == 128) SM_MF(4, 8);
+  else if (D == 128 && Dv == 64) SM_MF(4, 4);
+  else if (D == 64 && Dv == 128) SM_MF(2, 8);
+  else if (D == 32 && Dv == 32) SM_MF(1, 2);
+  else return 1;
+#undef SM_MF
   return (int)hipGetLastError();
 }
 

@@ -232,6 +232,9 @@ def pool_blocks(k_pages, v_pages, k_pool, v_pool, meta: RaggedMeta, pool: int) -
             b += 1
 
 
+ATTN_MFMA_MIN = int(__import__("os").environ.get("EDGELLM_ATTN_MFMA_MIN", "16"))
+
+
 def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages, v_pages, k_pool, v_pool,
                           meta: RaggedMeta, scale: float, window: Optional[int], pool: Optional[int]) -> torch.Tensor:
     """q [T, H, D] -> [T, H * Dv].  Query position i sees the tokens j with 0 <= i - j < window and
@@ -240,9 +243,15 @@ def window_pool_attention(q: torch.Tensor, gate: Optional[torch.Tensor], k_pages
     T, H, D = q.shape
     G, Dv = k_pages.shape[2], v_pages.shape[3]
     if _gpu(q):
+        # bf16 steps with a portion of ATTN_MFMA_MIN tokens or more: the MFMA kernel (64 query rows per
+        # workgroup); decode-sized steps and fp32: one workgroup per (token, kv head)
+        qtiles = 0
+        if q.dtype == torch.bfloat16 and meta.max_len >= ATTN_MFMA_MIN:
+            qtiles = sum((h[2] + 63) // 64 for h in meta.host)
         return _ext().sm_attention(q, gate, k_pages, v_pages, k_pool if pool else None, v_pool if pool else None,
                                    meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.page_table, float(scale),
-                                   int(window) if window is not None else 0, int(pool or 0), int(meta.max_keys))
+                                   int(window) if window is not None else 0, int(pool or 0), int(meta.max_keys),
+                                   meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n), int(qtiles))
     page = meta.page
     out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
     R = H // G

@@ -402,3 +402,74 @@ def test_greedy_generation_through_scheduler_and_server(tmp_path, dev):
             assert x is None or f.result(timeout=120)["tokens"] == x
     finally:
         srv.close()
+
+
+@pytest.mark.gpu
+def test_decode_graph_replays_match_eager(tmp_path):
+    """Decode steps through the captured graph (replayed many times, host work and other eager
+    steps between the replays, batch sizes changing) equal the same steps run eagerly."""
+    cfg = make_config(n_layers=2, loop=(0, 2, 2), window=12, pool=3, width=64, heads=4, kv_heads=1, dim=16, vdim=8)
+    w = make_weights(cfg, seed=21)
+    outs = {}
+    for graphs in (False, True):
+        model = load(tmp_path, cfg, w, "cuda", precision="bf16")
+        eng = RaggedEngine(model, 4 * 128, slots=4, use_graphs=graphs)
+        reqs = {r: tokens(90, cfg["vocab"], 30 + i) for i, r in enumerate("abc")}
+        got = []
+        got.append(eng.step([("a", reqs["a"][:20], [19]), ("b", reqs["b"][:3], [2])]).cpu())
+        at = {"a": 20, "b": 3, "c": 0}
+        for k in range(40):
+            live = ["a", "b"] if k < 10 or k > 25 else ["a", "b", "c"]
+            if k == 10:
+                got.append(eng.step([("c", reqs["c"][:7], [6])]).cpu())
+                at["c"] = 7
+            got.append(eng.step([(r, [reqs[r][at[r]]], [0]) for r in live]).cpu())
+            for r in live:
+                at[r] += 1
+        assert eng.graphs_used == graphs
+        outs[graphs] = torch.cat(got)
+    assert torch.allclose(outs[True], outs[False], atol=2e-2, rtol=2e-2)
+    assert (outs[True] - outs[False]).abs().max() < 0.05
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window,pool,H,G,D,Dv", [(40, 8, 4, 2, 32, 32), (100, 16, 2, 1, 64, 64), (None, None, 2, 2, 32, 32),
+                                                  (70, 3, 3, 1, 96, 96), (33, 70, 2, 2, 128, 64)])
+def test_attention_bf16_prompt_kernel(window, pool, H, G, D, Dv):
+    """The matrix-core prompt kernel (bf16 portions of 16 tokens or more): two sequences in the
+    same steps, portions that start and end inside pages, a planted far key, against the oracle on
+    the bf16-rounded inputs; decode-sized steps in between take the general kernel."""
+    dev = "cuda"
+    torch.manual_seed(4)
+    Ts = {0: 333, 2: 150}
+    rnd = lambda *s: torch.randn(*s).to(torch.bfloat16).double()
+    data, want = {}, {}
+    for s, T in Ts.items():
+        q, k, v = rnd(T, H, D), rnd(T, G, D), rnd(T, G, Dv)
+        k[5] = (k[5] * 3).to(torch.bfloat16).double()
+        q[T - 3] = (k[5, 0] * 0.5).to(torch.bfloat16).double()
+        v[5] = (v[5] + 4).to(torch.bfloat16).double()
+        data[s] = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], 1).to(torch.bfloat16).to(dev)
+        want[s] = oracle.window_pool_attention(q, k, v, D ** -0.5, window, pool)
+    cache = _attn_cache(G, D, Dv, window, pool, 12, dev, dtype=torch.bfloat16)
+    run = cache.run(0)
+    sizes, at, got, kk = (70, 1, 64, 17, 2, 130, 16), {s: 0 for s in Ts}, {s: [] for s in Ts}, 0
+    while any(at[s] < Ts[s] for s in Ts):
+        n = sizes[kk % len(sizes)]
+        kk += 1
+        seqs = [(s, at[s], min(n + 3 * (s == 2), Ts[s] - at[s])) for s in Ts if at[s] < Ts[s]]
+        meta = _meta(cache, seqs, dev)
+        proj = torch.cat([data[s][a:a + m] for s, a, m in seqs])
+        qq = seqmix.rope_paged_write(proj, meta, None, run.k, run.v, H, 0)
+        if window and pool:
+            seqmix.pool_blocks(run.k, run.v, run.k_pool, run.v_pool, meta, pool)
+        o = seqmix.window_pool_attention(qq, None, run.k, run.v, run.k_pool, run.v_pool, meta, D ** -0.5, window,
+                                         pool if window else None).cpu().double()
+        off = 0
+        for s, a, m in seqs:
+            got[s].append(o[off:off + m])
+            off += m
+            at[s] += m
+    for s, T in Ts.items():
+        g = torch.cat(got[s]).view(T, H, Dv)
+        assert torch.allclose(g, want[s], atol=3e-2, rtol=3e-2), (s, (g - want[s]).abs().max())
