@@ -187,7 +187,8 @@ template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float
 template <typename KT, int RMAX, int DVL, bool VEC>
 __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const KT* __restrict__ vbase, int cnt, int g,
                                            int G, int D, int Dv, int R, const float* q_s, float* s_s, int* row_s,
-                                           float* m_s, float* l_s, float* a_s, int rowidx, float (&acc)[RMAX][DVL]) {
+                                           float* m_s, float* l_s, float* a_s, int rowidx, float (&acc)[RMAX][VEC ? 8 : DVL]) {
+  constexpr int AW = VEC ? 8 : DVL;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // (A) scores
   {
@@ -246,27 +247,58 @@ __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const K
   for (int r = 0; r < RMAX; ++r) {
     const float al = r < R ? a_s[r] : 1.f;
 #pragma unroll
-    for (int dl = 0; dl < DVL; ++dl) acc[r][dl] *= al;
+    for (int dl = 0; dl < AW; ++dl) acc[r][dl] *= al;
   }
   // eight rows' loads are issued before their products (the walk is latency-bound otherwise)
   const int j1 = min(cnt, 64 * (wave + 1));
   constexpr int UN = 8;
-  for (int j = 64 * wave; j < j1; j += UN) {
-    float vv[UN][DVL];
+  if constexpr (VEC) {
+    // lane = (key of the round, 8 value coordinates): LPK lanes cover a row with one 16-byte (bf16) or
+    // two (fp32) loads each, 64 / LPK rows per round, UN rounds in flight; the lanes' partial sums over
+    // their keys are added up once, after the last chunk
+    constexpr int LPK = 8 * DVL, KPR = 64 / LPK;
+    const int dpart = lane % LPK, ksub = lane / LPK;
+    const bool live = dpart * 8 < Dv;
+    for (int j = 64 * wave; j < j1; j += UN * KPR) {
+      float vv[UN][8];
 #pragma unroll
-    for (int k = 0; k < UN; ++k) {
-      const KT* vr = vbase + ((size_t)row_s[min(j + k, j1 - 1)] * G + g) * Dv;
+      for (int k = 0; k < UN; ++k) {
+        const int jk = j + k * KPR + ksub;
+        if (live && jk < j1) load8<KT>(vbase + ((size_t)row_s[jk] * G + g) * Dv + dpart * 8, vv[k]);
+        else {
 #pragma unroll
-      for (int dl = 0; dl < DVL; ++dl) vv[k][dl] = lane + 64 * dl < Dv ? ldf<KT>(vr + lane + 64 * dl) : 0.f;
-    }
+          for (int e = 0; e < 8; ++e) vv[k][e] = 0.f;
+        }
+      }
 #pragma unroll
-    for (int k = 0; k < UN; ++k) {
-      if (j + k < j1) {
+      for (int k = 0; k < UN; ++k) {
+        const int jk = min(j + k * KPR + ksub, j1 - 1);     // rows past the end were loaded as zeros
 #pragma unroll
         for (int r = 0; r < RMAX; ++r) {
-          const float p = s_s[r * KC + j + k];
+          const float p = s_s[r * KC + jk];
 #pragma unroll
-          for (int dl = 0; dl < DVL; ++dl) acc[r][dl] += p * vv[k][dl];
+          for (int e = 0; e < 8; ++e) acc[r][e] += p * vv[k][e];
+        }
+      }
+    }
+  } else {
+    for (int j = 64 * wave; j < j1; j += UN) {
+      float vv[UN][DVL];
+#pragma unroll
+      for (int k = 0; k < UN; ++k) {
+        const KT* vr = vbase + ((size_t)row_s[min(j + k, j1 - 1)] * G + g) * Dv;
+#pragma unroll
+        for (int dl = 0; dl < DVL; ++dl) vv[k][dl] = lane + 64 * dl < Dv ? ldf<KT>(vr + lane + 64 * dl) : 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < UN; ++k) {
+        if (j + k < j1) {
+#pragma unroll
+          for (int r = 0; r < RMAX; ++r) {
+            const float p = s_s[r * KC + j + k];
+#pragma unroll
+            for (int dl = 0; dl < DVL; ++dl) acc[r][dl] += p * vv[k][dl];
+          }
         }
       }
     }
@@ -302,11 +334,12 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
   }
   for (int e = tid; e < RMAX * Dv; e += NT) red[e] = 0.f;
   if (tid < RMAX) { m_s[tid] = -INFINITY; l_s[tid] = 0.f; a_s[tid] = 1.f; }
-  float acc[RMAX][DVL];
+  constexpr int AW = VEC ? 8 : DVL;
+  float acc[RMAX][AW];
 #pragma unroll
   for (int r = 0; r < RMAX; ++r)
 #pragma unroll
-    for (int dl = 0; dl < DVL; ++dl) acc[r][dl] = 0.f;
+    for (int dl = 0; dl < AW; ++dl) acc[r][dl] = 0.f;
   __syncthreads();
   const int jlo = window > 0 ? max(0, i - window + 1) : 0;
   const int nt = i - jlo + 1;
@@ -322,13 +355,33 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
     attn_chunk<float, RMAX, DVL, VEC>(kb, vb, min(KC, nb - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
   }
   // sum the four waves' partial outputs, normalise, gate
+  if constexpr (VEC) {                                       // add up the lanes that walked different keys
+    constexpr int LPK = 8 * DVL;
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int o = LPK; o < 64; o <<= 1) acc[r][e] += __shfl_xor(acc[r][e], o, 64);
+  }
   for (int w = 0; w < NT / 64; ++w) {
     if (wave == w) {
+      if constexpr (VEC) {
+        constexpr int LPK = 8 * DVL;
+        if (lane < LPK && lane * 8 < Dv) {
 #pragma unroll
-      for (int r = 0; r < RMAX; ++r)
+          for (int r = 0; r < RMAX; ++r)
 #pragma unroll
-        for (int dl = 0; dl < DVL; ++dl)
-          if (r < R && lane + 64 * dl < Dv) red[r * Dv + lane + 64 * dl] += acc[r][dl];
+            for (int e = 0; e < 8; ++e)
+              if (r < R) red[r * Dv + lane * 8 + e] += acc[r][e];
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+          for (int dl = 0; dl < DVL; ++dl)
+            if (r < R && lane + 64 * dl < Dv) red[r * Dv + lane + 64 * dl] += acc[r][dl];
+      }
     }
     __syncthreads();
   }
@@ -900,7 +953,7 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
   const size_t lds = sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 3 * rmax) +
                      sizeof(int) * KC;
   if (lds > 64 * 1024) return -3;
-  const bool vec = D % 8 == 0;
+  const bool vec = D % 8 == 0 && Dv % 8 == 0;
 #define SM_ATT_V(RM, DL, V)                                                                                         \
   SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL, V>), dim3(rows, G * nsp), dim3(NT), lds, st, (const T*)q,         \
                                (const T*)gate, gate_ld, (const T*)kp, (const T*)vp, kb, vb, tok_seq, tok_pos,       \
@@ -918,7 +971,8 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
     case 8: SM_ATT(8, DL); break;    \
     default: SM_ATT(16, DL); break;  \
   }
-  if (Dv <= 128) { SM_ATT_R(2); }
+  if (Dv <= 64) { SM_ATT_R(1); }
+  else if (Dv <= 128) { SM_ATT_R(2); }
   else { SM_ATT_R(4); }
 #undef SM_ATT_R
 #undef SM_ATT
