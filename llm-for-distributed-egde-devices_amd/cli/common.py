@@ -97,6 +97,13 @@ def build_generator(model, rt: dict, max_batch: int = 1):
     from ..engine import Generator
     from ..engine.kv_cache import resolve_kv_dtype
     max_seq = rt.get("max_seq", 2048)
+    if getattr(model, "ragged", False):
+        # layer-spec models: paged cache + ragged steps (prompt portions beside decode tokens); the
+        # pool holds max_batch sequences of max_seq tokens, prompts are fed in --prefill_chunk portions
+        from ..engine.ragged import RaggedGenerator
+        assert rt.get("headinfer_heads") is None, "HeadInfer offload runs on the row-cache models"
+        return RaggedGenerator(model, max_batch=max(max_batch, 1), max_seq=max_seq,
+                               prefill_chunk=int(rt.get("prefill_chunk") or 512))
     h_on = rt.get("headinfer_heads")
     if h_on is not None and h_on < model.cfg.num_kv_heads:
         assert not hasattr(model, "make_kv"), "HeadInfer offload runs on a single-device model"

@@ -73,6 +73,16 @@ class HybridLM(nn.Module):
     def device(self):
         return self.embed.device
 
+    @torch.no_grad()
+    def confidence(self, ids) -> float:
+        """mean over the text's tokens of max softmax probability (eval.metrics.confidence_score):
+        one ragged prompt pass through a cache of its own."""
+        from .. import ops
+        from ..engine.ragged import RaggedEngine
+        eng = RaggedEngine(self, len(ids), slots=1, use_graphs=False)
+        logits = eng.step([("c", list(ids), list(range(len(ids))))])
+        return float(ops.max_softmax_prob(logits).mean())
+
     def run_specs(self):
         """The LayerSpec of every run, in order (sizes the paged cache)."""
         return [self.cfg.layer_specs[i] for i, _ in self.runs]

@@ -473,3 +473,31 @@ def test_attention_bf16_prompt_kernel(window, pool, H, G, D, Dv):
     for s, T in Ts.items():
         g = torch.cat(got[s]).view(T, H, Dv)
         assert torch.allclose(g, want[s], atol=3e-2, rtol=3e-2), (s, (g - want[s]).abs().max())
+
+
+def test_evaluate_cli_runs_a_nudadra_checkpoint(tmp_path):
+    """The evaluation command line on a checkpoint folder of this design (vocabulary wide enough
+    for the byte tokenizer): loader by config.json, paged engine, the reference's sampling
+    configuration, the confidence metric through the model's own prompt pass."""
+    from safetensors.torch import save_file
+    from edgellm.cli import evaluate
+    cfg = make_config(vocab=300, n_layers=2, loop=(1, 2, 2), window=20, pool=4)
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file(make_weights(cfg, seed=3), str(d / "model.safetensors"))
+    y = tmp_path / "c.yaml"
+    y.write_text(f"""
+max_new_tokens: 4
+temperature: 0.7
+top_k: 50
+top_p: 0.9
+repetition_penalty: 1.1
+dataset_name: sentence-transformers/natural-questions
+dataset_split: train[:2]
+embedder_model: "none"
+models: ["{d}"]
+""")
+    out = evaluate.main(["--config", str(y), "--devices", "cpu", "--num_samples", "2", "--max_seq", "256",
+                         "--batch_size", "2", "--prefill_chunk", "16", "--precision", "fp32"])
+    assert out[str(d)]["tps"] > 0 and 0 < out[str(d)]["confidence"] <= 1
