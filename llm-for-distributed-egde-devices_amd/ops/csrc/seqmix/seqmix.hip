@@ -20,6 +20,24 @@ template <typename T> __device__ __forceinline__ void stf(T* p, float v);
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
 
+template <typename KT> __device__ __forceinline__ void load8(const KT* p, float* f);
+template <> __device__ __forceinline__ void load8<float>(const float* p, float* f) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float* f) {
+  unpack8(*reinterpret_cast<const uint4*>(p), f);
+}
+
+template <typename T> __device__ __forceinline__ void store8(T* p, const float* f);
+template <> __device__ __forceinline__ void store8<float>(float* p, const float* f) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(f[4], f[5], f[6], f[7]);
+}
+template <> __device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float* f) {
+  *reinterpret_cast<uint4*>(p) = pack8(f);
+}
+
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float siluf_(float x) { return x * sigmoidf_(x); }
 
@@ -47,12 +65,23 @@ __global__ void __launch_bounds__(NT) scalar_norm_kernel(const float* __restrict
   for (int c = threadIdx.x; c < W; c += NT) stf<T>(y + (size_t)blockIdx.x * W + c, xr[c] * r);
 }
 
-template <typename T>
+// VEC: eight columns per thread through 16-byte accesses (ld, c0, C multiples of 8)
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) relu2_kernel(const T* __restrict__ u, int ld, int c0, T* __restrict__ y, int C) {
   const int t = blockIdx.x;
-  for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
-    const float v = fmaxf(ldf<T>(u + (size_t)t * ld + c0 + c), 0.f);
-    stf<T>(y + (size_t)t * C + c, v * v);
+  if constexpr (VEC) {
+    for (int c = (blockIdx.y * NT + threadIdx.x) * 8; c < C; c += NT * gridDim.y * 8) {
+      float f[8];
+      load8<T>(u + (size_t)t * ld + c0 + c, f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float v = fmaxf(f[e], 0.f); f[e] = v * v; }
+      store8<T>(y + (size_t)t * C + c, f);
+    }
+  } else {
+    for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
+      const float v = fmaxf(ldf<T>(u + (size_t)t * ld + c0 + c), 0.f);
+      stf<T>(y + (size_t)t * C + c, v * v);
+    }
   }
 }
 
@@ -174,15 +203,6 @@ __global__ void __launch_bounds__(NT) pool_kernel(const T* __restrict__ kp, cons
 // chunk with lane = value coordinate (coalesced row reads).  Tokens of the window first, then the
 // pooled blocks (fp32 rows): one softmax over both.
 constexpr int KC = 256;
-
-template <typename KT> __device__ __forceinline__ void load8(const KT* p, float* f);
-template <> __device__ __forceinline__ void load8<float>(const float* p, float* f) {
-  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
-  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
-}
-template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float* f) {
-  unpack8(*reinterpret_cast<const uint4*>(p), f);
-}
 
 template <typename KT, int RMAX, int DVL, bool VEC>
 __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const KT* __restrict__ vbase, int cnt, int g,
@@ -447,38 +467,55 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
   const int nbmax = (window > 0 && pool > 0 && imax - window + 1 > 0) ? (imax - window + 1) / pool : 0;
   const int tok_tiles = imax / MK - jlo / MK + 1, ntiles = tok_tiles + (nbmax + MK - 1) / MK;
 
+  // a tile's rows travel global -> registers while the tile before it computes, registers -> LDS
+  // between the two barriers
+  static_assert(DV % 2 == 0, "value chunks per thread");
+  constexpr int KL = DK, VL = DV / 2;                        // 16-byte chunks per thread per tile
+  uint4 kreg[KL], vreg[VL];
+  auto load_tile = [&](int tile) {
+    const bool tok = tile < tok_tiles;
+    const int base = tok ? (jlo / MK + tile) * MK : (tile - tok_tiles) * MK;
+    const size_t prow = tok ? (size_t)pt[base / MK] * MK : 0;
+#pragma unroll
+    for (int i = 0; i < KL + VL; ++i) {
+      const bool isk = i < KL;
+      const int e = tid + (isk ? i : i - KL) * NT, cpr = isk ? D / 8 : Dv / 8;
+      const int r = e / cpr, c = e % cpr;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (tok) {
+        v = isk ? *reinterpret_cast<const uint4*>(kp + ((prow + r) * G + g) * D + c * 8)
+                : *reinterpret_cast<const uint4*>(vp + ((prow + r) * G + g) * Dv + c * 8);
+      } else if (base + r < nbmax) {
+        const int p0 = (base + r) * pool;
+        const size_t row = ((size_t)pt[p0 / MK] * PB + (p0 % MK) / pool) * G + g;
+        float f[8];
+        load8<float>(isk ? kb + row * D + c * 8 : vb + row * Dv + c * 8, f);
+        v = pack8(f);
+      }
+      if (isk) kreg[i] = v;
+      else vreg[i - KL] = v;
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < KL; ++i) {
+      const int e = tid + i * NT;
+      *reinterpret_cast<uint4*>(k_lds + (e / (D / 8)) * KS + (e % (D / 8)) * 16) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VL; ++i) {
+      const int e = tid + i * NT;
+      *reinterpret_cast<uint4*>(v_lds + (e / (Dv / 8)) * VS + (e % (Dv / 8)) * 16) = vreg[i];
+    }
+  };
+  if (ntiles > 0) load_tile(0);
   for (int tile = 0; tile < ntiles; ++tile) {
     const bool tok = tile < tok_tiles;
     const int base = tok ? (jlo / MK + tile) * MK : (tile - tok_tiles) * MK;   // first position / block of the tile
     __syncthreads();                                         // every wave is done with the previous tile
-    if (tok) {
-      const size_t prow = (size_t)pt[base / MK] * MK;
-      for (int e = tid; e < MK * (D / 8); e += NT) {
-        const int r = e / (D / 8), c = e % (D / 8);
-        *reinterpret_cast<uint4*>(k_lds + r * KS + c * 16) =
-            *reinterpret_cast<const uint4*>(kp + ((prow + r) * G + g) * D + c * 8);
-      }
-      for (int e = tid; e < MK * (Dv / 8); e += NT) {
-        const int r = e / (Dv / 8), c = e % (Dv / 8);
-        *reinterpret_cast<uint4*>(v_lds + r * VS + c * 16) =
-            *reinterpret_cast<const uint4*>(vp + ((prow + r) * G + g) * Dv + c * 8);
-      }
-    } else {
-      for (int e = tid; e < MK * (D / 8 + Dv / 8); e += NT) {
-        const int r = e / (D / 8 + Dv / 8), c = e % (D / 8 + Dv / 8);
-        const int b = base + r;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (b < nbmax) {
-          const int p0 = b * pool;
-          const size_t row = ((size_t)pt[p0 / MK] * PB + (p0 % MK) / pool) * G + g;
-          float f[8];
-          load8<float>(c < D / 8 ? kb + row * D + c * 8 : vb + row * Dv + (c - D / 8) * 8, f);
-          v = pack8(f);
-        }
-        *reinterpret_cast<uint4*>(c < D / 8 ? k_lds + r * KS + c * 16 : v_lds + r * VS + (c - D / 8) * 16) = v;
-      }
-    }
+    store_tile();
     __syncthreads();
+    if (tile + 1 < ntiles) load_tile(tile + 1);
     v4f sc[4];
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
@@ -562,7 +599,7 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
 // ---------------------------------------------------------------------------------- convolution
 constexpr int MAX_TAPS = 16;
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) conv_kernel(const T* __restrict__ u, int ld, int c0, int C,
                                                   const float* __restrict__ w, const float* __restrict__ bias,
                                                   const T* __restrict__ state, const int* __restrict__ tok_seq,
@@ -572,16 +609,36 @@ __global__ void __launch_bounds__(NT) conv_kernel(const T* __restrict__ u, int l
   const int t = blockIdx.x, s = tok_seq[t];
   const int pos = tok_pos[t], start = seq_start[s], off = seq_off[s];
   const T* st = state + (size_t)seq_slot[s] * (taps - 1) * C;
-  for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
-    float acc = bias[c];
-    for (int k = 0; k < taps; ++k) {
-      const int p = pos - (taps - 1) + k;
-      float x = 0.f;
-      if (p >= start) x = ldf<T>(u + (size_t)(off + p - start) * ld + c0 + c);
-      else if (p >= 0) x = ldf<T>(st + (size_t)(p - (start - (taps - 1))) * C + c);
-      acc += w[c * taps + k] * x;
+  if constexpr (VEC) {                                       // eight channels per thread (ld, c0, C multiples of 8)
+    for (int c = (blockIdx.y * NT + threadIdx.x) * 8; c < C; c += NT * gridDim.y * 8) {
+      float acc[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = bias[c + e];
+      for (int k = 0; k < taps; ++k) {
+        const int p = pos - (taps - 1) + k;
+        if (p < 0) continue;
+        float x[8];
+        if (p >= start) load8<T>(u + (size_t)(off + p - start) * ld + c0 + c, x);
+        else load8<T>(st + (size_t)(p - (start - (taps - 1))) * C + c, x);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += w[(c + e) * taps + k] * x[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
+      store8<T>(out + (size_t)t * C + c, acc);
     }
-    stf<T>(out + (size_t)t * C + c, siluf_(acc));
+  } else {
+    for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
+      float acc = bias[c];
+      for (int k = 0; k < taps; ++k) {
+        const int p = pos - (taps - 1) + k;
+        float x = 0.f;
+        if (p >= start) x = ldf<T>(u + (size_t)(off + p - start) * ld + c0 + c);
+        else if (p >= 0) x = ldf<T>(st + (size_t)(p - (start - (taps - 1))) * C + c);
+        acc += w[c * taps + k] * x;
+      }
+      stf<T>(out + (size_t)t * C + c, siluf_(acc));
+    }
   }
 }
 
@@ -894,8 +951,13 @@ int edge_sm_scalar_norm(const float* x, const float* gain, void* y, int rows, in
 
 int edge_sm_relu2(const void* u, int ld, int c0, void* y, int rows, int C, int f32, hipStream_t st) {
   if (rows == 0 || C == 0) return 0;
-  const int gy = (C + NT * 4 - 1) / (NT * 4);
-  SM_T(f32, hipLaunchKernelGGL(relu2_kernel<T>, dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, (T*)y, C));
+  if (ld % 8 == 0 && c0 % 8 == 0 && C % 8 == 0) {
+    const int gy = (C / 8 + NT - 1) / NT;
+    SM_T(f32, hipLaunchKernelGGL((relu2_kernel<T, true>), dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, (T*)y, C));
+  } else {
+    const int gy = (C + NT * 4 - 1) / (NT * 4);
+    SM_T(f32, hipLaunchKernelGGL((relu2_kernel<T, false>), dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, (T*)y, C));
+  }
   return (int)hipGetLastError();
 }
 
@@ -987,8 +1049,13 @@ int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, cons
   if (rows == 0) return 0;
   if (taps < 1 || taps > MAX_TAPS) return -2;
   const int gy = (C + NT - 1) / NT;
-  SM_T(f32, hipLaunchKernelGGL(conv_kernel<T>, dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, w, bias,
-                               (const T*)state, tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps));
+  if (ld % 8 == 0 && c0 % 8 == 0 && C % 8 == 0)
+    SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, true>), dim3(rows, (C / 8 + NT - 1) / NT), dim3(NT), 0, st,
+                                 (const T*)u, ld, c0, C, w, bias, (const T*)state, tok_seq, tok_pos, seq_slot,
+                                 seq_start, seq_off, (T*)out, taps));
+  else
+    SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, false>), dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, w,
+                                 bias, (const T*)state, tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps));
   if (taps > 1)
     SM_T(f32, hipLaunchKernelGGL(conv_state_kernel<T>, dim3(n, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, (T*)state,
                                  seq_slot, seq_start, seq_len, seq_off, taps));

@@ -202,7 +202,8 @@ def test_attention_op_portions_and_a_far_key(dev, window, pool, H, G, D, Dv, pag
 @pytest.mark.parametrize("dev", DEVS)
 @pytest.mark.parametrize("Hs,P,N,groups,taps,sizes", [
     (2, 4, 3, 1, 4, (1, 2, 3, 4, 5)), (4, 8, 16, 2, 2, (1, 2, 3, 4, 5)), (3, 5, 20, 3, 5, (1, 2, 3, 4, 5)),
-    (1, 70, 33, 1, 3, (1, 2, 3, 4, 5)), (2, 70, 67, 2, 4, (64, 1, 33, 65, 2, 130)), (3, 16, 8, 1, 3, (40, 100, 7))])
+    (1, 70, 33, 1, 3, (1, 2, 3, 4, 5)), (2, 70, 67, 2, 4, (64, 1, 33, 65, 2, 130)), (3, 16, 8, 1, 3, (40, 100, 7)),
+    (8, 8, 8, 1, 4, (1, 2, 3, 4, 5)), (8, 8, 8, 1, 4, (40, 100, 7))])
 def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps, sizes):
     """Convolution tail and state matrix carried over portions of ``sizes`` tokens (short ones step
     token by token, long ones take the chunked form; chunk borders inside and at the end of a
