@@ -20,6 +20,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -124,7 +125,7 @@ class RaggedEngine:
             start = self.cache.lens[slot]
             self.cache.extend(slot, start + len(toks))
             seqs.append((slot, start, len(toks)))
-            ids.extend(int(t) for t in toks)
+            ids.extend(toks)
             rows.extend(off + int(w) for w in want)
             off += len(toks)
         if not seqs:
@@ -140,8 +141,11 @@ class RaggedEngine:
                 return out.clone()
             return out.index_select(0, torch.tensor(rows, dtype=torch.long, device=self.device))
         meta = RaggedMeta.build(seqs, self.cache.page_table, self.page, self.device)
-        ids_t = torch.tensor(ids, dtype=torch.long, device=self.device)
-        rows_t = torch.tensor(rows, dtype=torch.long, device=self.device)
+        ids_t = torch.from_numpy(np.asarray(ids, dtype=np.int64))
+        rows_t = torch.from_numpy(np.asarray(rows, dtype=np.int64))
+        if self.device.type == "cuda":
+            ids_t = ids_t.pin_memory().to(self.device, non_blocking=True)
+            rows_t = rows_t.pin_memory().to(self.device, non_blocking=True)
         with trace_range(f"ragged.step.n{meta.n}.T{meta.T}"):
             return self.model(ids_t, meta, self.cache, rows_t, taps)
 

@@ -27,7 +27,8 @@ int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, co
 int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
-                      int window, int pool, int f32, hipStream_t st);
+                      int window, int pool, int f32, int nsplit, float* part, hipStream_t st);
+size_t edge_sm_attention_part_floats(int rows, int H, int G, int Dv, int nsplit);
 int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp,
                            const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
                            const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
@@ -36,7 +37,7 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
 int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
                       const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
                       const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
-                      hipStream_t st);
+                      int max_len, hipStream_t st);
 int edge_sm_ssd_scan(const void* xbc, int Cx, const void* u, int ld, int dt0, const float* dt_bias, const float* A_log,
                      const float* Dp, float* state, const int* seq_slot, const int* seq_start, const int* seq_len,
                      const int* seq_off, float* y, int n, int Hs, int P, int N, int groups, int f32, hipStream_t st);
@@ -249,18 +250,30 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
       return out;
     }
   }
+  // few queries over many keys (decode steps): split every query's keys over several workgroups
+  int nsplit = 1;
+  {
+    const int64_t vis = (window > 0 ? std::min<int64_t>(window, max_keys) : max_keys) + (PB ? max_keys / pool : 0);
+    const int64_t chunks = (vis + 255) / 256;
+    if (T * G <= 64 && chunks > 1) nsplit = (int)std::min<int64_t>(chunks, 8);
+  }
+  at::Tensor part;
+  if (nsplit > 1)
+    part = at::empty({(int64_t)edge_sm_attention_part_floats((int)T, (int)H, (int)G, (int)Dv, nsplit)},
+                     q.options().dtype(at::kFloat));
   check(edge_sm_attention(q.data_ptr(), gate ? gate->data_ptr() : nullptr, gate_ld, kp.data_ptr(), vp.data_ptr(),
                           PB ? kb->data_ptr<float>() : nullptr, PB ? vb->data_ptr<float>() : nullptr,
                           tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),
                           ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)T, (int)H, (int)G, (int)D, (int)Dv,
-                          (int)page, PB, (float)scale, (int)window, PB ? (int)pool : 0, f32(q), stream()), "sm_attention");
+                          (int)page, PB, (float)scale, (int)window, PB ? (int)pool : 0, f32(q), nsplit,
+                          nsplit > 1 ? part.data_ptr<float>() : nullptr, stream()), "sm_attention");
   return out;
 }
 
 at::Tensor sm_conv_silu(const at::Tensor& u, int64_t c0, int64_t C, const at::Tensor& w, const at::Tensor& bias,
                         at::Tensor& state, const at::Tensor& tok_seq, const at::Tensor& tok_pos,
                         const at::Tensor& seq_slot, const at::Tensor& seq_start, const at::Tensor& seq_len,
-                        const at::Tensor& seq_off, int64_t n) {
+                        const at::Tensor& seq_off, int64_t n, int64_t max_len) {
   const int ld = row_ld(u, "u");
   chk_f32(w, "conv weight");
   chk_f32(bias, "conv bias");
@@ -276,7 +289,7 @@ at::Tensor sm_conv_silu(const at::Tensor& u, int64_t c0, int64_t C, const at::Te
   check(edge_sm_conv_silu(u.data_ptr(), ld, (int)c0, (int)C, w.data_ptr<float>(), bias.data_ptr<float>(), state.data_ptr(),
                           tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),
                           seq_start.data_ptr<int>(), seq_len.data_ptr<int>(), seq_off.data_ptr<int>(), out.data_ptr(),
-                          (int)T, (int)n, (int)taps, f32(u), stream()), "sm_conv_silu");
+                          (int)T, (int)n, (int)taps, f32(u), (int)max_len, stream()), "sm_conv_silu");
   return out;
 }
 

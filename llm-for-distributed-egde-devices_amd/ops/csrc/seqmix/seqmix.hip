@@ -333,7 +333,8 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
                                                   const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                                   const int* __restrict__ seq_slot, const int* __restrict__ ptab,
                                                   int ptab_ld, T* __restrict__ out, int H, int G, int D, int Dv,
-                                                  int page, int PB, float scale, int window, int pool, int nsp) {
+                                                  int page, int PB, float scale, int window, int pool, int nsp, int nsplit,
+                                                  float* __restrict__ part) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   // more than RMAX query heads per kv head: nsp workgroups share the kv head, RMAX heads each
   const int t = blockIdx.x, g = blockIdx.y / nsp, r0 = (blockIdx.y % nsp) * RMAX;
@@ -364,12 +365,18 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
   const int jlo = window > 0 ? max(0, i - window + 1) : 0;
   const int nt = i - jlo + 1;
   const int nb = (window > 0 && pool > 0 && i - window + 1 > 0) ? (i - window + 1) / pool : 0;
-  for (int c0 = 0; c0 < nt; c0 += KC) {
+  // key chunks [ci0, ci1) of this query belong to this workgroup (blockIdx.z of nsplit; 1: all of them)
+  const int nchunks = (nt + KC - 1) / KC + (nb + KC - 1) / KC, cps = (nchunks + nsplit - 1) / nsplit;
+  const int ci0 = blockIdx.z * cps, ci1 = min(nchunks, ci0 + cps);
+  int ci = 0;
+  for (int c0 = 0; c0 < nt; c0 += KC, ++ci) {
+    if (ci < ci0 || ci >= ci1) continue;
     const int j = jlo + c0 + tid;
     const int rowidx = c0 + tid < nt ? pt[j / page] * page + j % page : 0;
     attn_chunk<T, RMAX, DVL, VEC>(kp, vp, min(KC, nt - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
   }
-  for (int c0 = 0; c0 < nb; c0 += KC) {
+  for (int c0 = 0; c0 < nb; c0 += KC, ++ci) {
+    if (ci < ci0 || ci >= ci1) continue;
     const int p0 = (c0 + tid) * pool;
     const int rowidx = c0 + tid < nb ? pt[p0 / page] * PB + (p0 % page) / pool : 0;
     attn_chunk<float, RMAX, DVL, VEC>(kb, vb, min(KC, nb - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
@@ -405,11 +412,43 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
     }
     __syncthreads();
   }
+  if (nsplit > 1) {                                          // unnormalised sums, running max and sum per head
+    float* dst = part + (((size_t)t * gridDim.y + blockIdx.y) * nsplit + blockIdx.z) * (RMAX * (Dv + 2));
+    for (int e = tid; e < R * Dv; e += NT) dst[e] = red[e];
+    if (tid < R) { dst[RMAX * Dv + tid] = m_s[tid]; dst[RMAX * Dv + RMAX + tid] = l_s[tid]; }
+    return;
+  }
   for (int e = tid; e < R * Dv; e += NT) {
     const int r = e / Dv, h = hq0 + r;
     float o = red[e] / l_s[r];
     if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + h));
     stf<T>(out + ((size_t)t * H + h) * Dv + e % Dv, o);
+  }
+}
+
+
+// sums the key-split partial results of attn_kernel: out = sum_z e^{m_z - M} acc_z / sum_z e^{m_z - M} l_z
+template <typename T>
+__global__ void __launch_bounds__(NT) attn_merge_kernel(const float* __restrict__ part, const T* __restrict__ gate,
+                                                        int gate_ld, T* __restrict__ out, int H, int G, int Dv, int nsp,
+                                                        int nsplit, int rmax) {
+  const int t = blockIdx.x, g = blockIdx.y / nsp, r0 = (blockIdx.y % nsp) * rmax;
+  const int R = min(rmax, H / G - r0), hq0 = g * (H / G) + r0, stride = rmax * (Dv + 2);
+  const float* src = part + ((size_t)t * gridDim.y + blockIdx.y) * nsplit * stride;
+  for (int e = threadIdx.x; e < R * Dv; e += NT) {
+    const int r = e / Dv;
+    float M = -INFINITY;
+    for (int z = 0; z < nsplit; ++z) M = fmaxf(M, src[z * stride + rmax * Dv + r]);
+    float acc = 0.f, l = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float mz = src[z * stride + rmax * Dv + r];
+      const float wz = mz == -INFINITY ? 0.f : expf(mz - M);
+      acc += wz * src[z * stride + e];
+      l += wz * src[z * stride + rmax * Dv + rmax + r];
+    }
+    float o = acc / l;
+    if (gate) o *= sigmoidf_(ldf<T>(gate + (size_t)t * gate_ld + hq0 + r));
+    stf<T>(out + ((size_t)t * H + hq0 + r) * Dv + e % Dv, o);
   }
 }
 
@@ -602,26 +641,42 @@ constexpr int MAX_TAPS = 16;
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) conv_kernel(const T* __restrict__ u, int ld, int c0, int C,
                                                   const float* __restrict__ w, const float* __restrict__ bias,
-                                                  const T* __restrict__ state, const int* __restrict__ tok_seq,
+                                                  const T* state, const int* __restrict__ tok_seq,
                                                   const int* __restrict__ tok_pos, const int* __restrict__ seq_slot,
                                                   const int* __restrict__ seq_start, const int* __restrict__ seq_off,
-                                                  T* __restrict__ out, int taps) {
+                                                  T* __restrict__ out, int taps, T* state_w) {
+  // state_w (steps in which every sequence brings one token: the thread of (token, channel) is the only
+  // reader of that channel's tail): the tail is shifted here and no second launch follows
   const int t = blockIdx.x, s = tok_seq[t];
   const int pos = tok_pos[t], start = seq_start[s], off = seq_off[s];
   const T* st = state + (size_t)seq_slot[s] * (taps - 1) * C;
+  T* stw = state_w ? state_w + (size_t)seq_slot[s] * (taps - 1) * C : nullptr;
   if constexpr (VEC) {                                       // eight channels per thread (ld, c0, C multiples of 8)
     for (int c = (blockIdx.y * NT + threadIdx.x) * 8; c < C; c += NT * gridDim.y * 8) {
       float acc[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = bias[c + e];
-      for (int k = 0; k < taps; ++k) {
-        const int p = pos - (taps - 1) + k;
-        if (p < 0) continue;
-        float x[8];
-        if (p >= start) load8<T>(u + (size_t)(off + p - start) * ld + c0 + c, x);
-        else load8<T>(st + (size_t)(p - (start - (taps - 1))) * C + c, x);
+      for (int k0 = 0; k0 < taps; k0 += 4) {                 // four taps' rows in flight
+        float x[4][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] += w[(c + e) * taps + k] * x[e];
+        for (int kk = 0; kk < 4; ++kk) {
+          const int k = k0 + kk, p = pos - (taps - 1) + k;
+          if (k < taps && p >= start) load8<T>(u + (size_t)(off + p - start) * ld + c0 + c, x[kk]);
+          else if (k < taps && p >= 0) load8<T>(st + (size_t)(p - (start - (taps - 1))) * C + c, x[kk]);
+          else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[kk][e] = 0.f;
+          }
+        }
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          if (k0 + kk < taps) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += w[(c + e) * taps + k0 + kk] * x[kk][e];
+            // the new tail = inputs of positions pos - (taps - 2) .. pos = taps 1 .. taps - 1 of this window
+            if (stw && k0 + kk >= 1) store8<T>(stw + (size_t)(k0 + kk - 1) * C + c, x[kk]);
+          }
+        }
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
@@ -636,6 +691,7 @@ __global__ void __launch_bounds__(NT) conv_kernel(const T* __restrict__ u, int l
         if (p >= start) x = ldf<T>(u + (size_t)(off + p - start) * ld + c0 + c);
         else if (p >= 0) x = ldf<T>(st + (size_t)(p - (start - (taps - 1))) * C + c);
         acc += w[c * taps + k] * x;
+        if (stw && k >= 1) stf<T>(stw + (size_t)(k - 1) * C + c, x);
       }
       stf<T>(out + (size_t)t * C + c, siluf_(acc));
     }
@@ -1003,23 +1059,31 @@ int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, co
   return (int)hipGetLastError();
 }
 
+// nsplit > 1: the keys of every query are walked by nsplit workgroups (decode steps: few queries, long
+// windows); part = fp32 scratch [rows, G * nsp, nsplit, rmax * (Dv + 2)] (edge_sm_attention_part_floats)
+size_t edge_sm_attention_part_floats(int rows, int H, int G, int Dv, int nsplit) {
+  const int R = H / G, rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16, nsp = (R + rmax - 1) / rmax;
+  return (size_t)rows * G * nsp * nsplit * rmax * (Dv + 2);
+}
+
 int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
-                      int window, int pool, int f32, hipStream_t st) {
+                      int window, int pool, int f32, int nsplit, float* part, hipStream_t st) {
   if (rows == 0) return 0;
   if (G <= 0 || H % G || Dv > 256) return -2;
   const int R = H / G;
   const int rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16;
   const int nsp = (R + rmax - 1) / rmax;
+  if (nsplit < 1 || (nsplit > 1 && !part)) return -2;
   const size_t lds = sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 3 * rmax) +
                      sizeof(int) * KC;
   if (lds > 64 * 1024) return -3;
   const bool vec = D % 8 == 0 && Dv % 8 == 0;
 #define SM_ATT_V(RM, DL, V)                                                                                         \
-  SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL, V>), dim3(rows, G * nsp), dim3(NT), lds, st, (const T*)q,         \
+  SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL, V>), dim3(rows, G * nsp, nsplit), dim3(NT), lds, st, (const T*)q,         \
                                (const T*)gate, gate_ld, (const T*)kp, (const T*)vp, kb, vb, tok_seq, tok_pos,       \
-                               seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool, nsp))
+                               seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool, nsp, nsplit, part))
 #define SM_ATT(RM, DL)               \
   do {                               \
     if (vec) SM_ATT_V(RM, DL, true); \
@@ -1039,24 +1103,29 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
 #undef SM_ATT_R
 #undef SM_ATT
 #undef SM_ATT_V
+  if (nsplit > 1)
+    SM_T(f32, hipLaunchKernelGGL(attn_merge_kernel<T>, dim3(rows, G * nsp), dim3(NT), 0, st, part, (const T*)gate, gate_ld,
+                                 (T*)out, H, G, Dv, nsp, nsplit, rmax));
   return (int)hipGetLastError();
 }
 
 int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
                       const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
                       const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
-                      hipStream_t st) {
+                      int max_len, hipStream_t st) {
   if (rows == 0) return 0;
   if (taps < 1 || taps > MAX_TAPS) return -2;
+  const bool one = max_len == 1 && taps > 1;                 // every sequence brings one token
   const int gy = (C + NT - 1) / NT;
   if (ld % 8 == 0 && c0 % 8 == 0 && C % 8 == 0)
     SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, true>), dim3(rows, (C / 8 + NT - 1) / NT), dim3(NT), 0, st,
                                  (const T*)u, ld, c0, C, w, bias, (const T*)state, tok_seq, tok_pos, seq_slot,
-                                 seq_start, seq_off, (T*)out, taps));
+                                 seq_start, seq_off, (T*)out, taps, one ? (T*)state : (T*)nullptr));
   else
     SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, false>), dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, w,
-                                 bias, (const T*)state, tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps));
-  if (taps > 1)
+                                 bias, (const T*)state, tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps,
+                                 one ? (T*)state : (T*)nullptr));
+  if (taps > 1 && !one)
     SM_T(f32, hipLaunchKernelGGL(conv_state_kernel<T>, dim3(n, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, (T*)state,
                                  seq_slot, seq_start, seq_len, seq_off, taps));
   return (int)hipGetLastError();

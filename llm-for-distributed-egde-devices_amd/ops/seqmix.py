@@ -77,17 +77,17 @@ class RaggedMeta:
     @classmethod
     def build(cls, seqs: List[Tuple[int, int, int]], page_table: torch.Tensor, page: int, device) -> "RaggedMeta":
         """``seqs``: (slot, start, len) per sequence, in flat-row order.  One host -> device copy."""
+        import numpy as np
         host, off = [], 0
         for slot, start, n in seqs:
             host.append((slot, start, n, off))
             off += n
         T, n = off, len(seqs)
-        flat = [h[0] for h in host] + [h[1] for h in host] + [h[2] for h in host] + [h[3] for h in host]
-        for i, (_, start, ln, _) in enumerate(host):
-            flat += [i] * ln
-        for (_, start, ln, _) in host:
-            flat += list(range(start, start + ln))
-        buf = torch.tensor(flat, dtype=torch.int32)
+        h = np.asarray(host, dtype=np.int32).reshape(n, 4)
+        lens = h[:, 2]
+        tok_seq = np.repeat(np.arange(n, dtype=np.int32), lens)
+        tok_pos = np.arange(T, dtype=np.int32) - np.repeat(h[:, 3] - h[:, 1], lens)
+        buf = torch.from_numpy(np.concatenate([h[:, 0], h[:, 1], h[:, 2], h[:, 3], tok_seq, tok_pos]))
         if torch.device(device).type == "cuda":
             buf = buf.pin_memory().to(device, non_blocking=True)
         s = lambda a, b: buf[a:b]
@@ -299,7 +299,7 @@ def conv_silu(u: torch.Tensor, c0: int, C: int, weight: torch.Tensor, bias: torc
     taps = weight.shape[1]
     if _gpu(u):
         out = _ext().sm_conv_silu(u, int(c0), int(C), weight, bias, state, meta.tok_seq, meta.tok_pos, meta.seq_slot,
-                                  meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n))
+                                  meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n), int(meta.max_len))
         return out
     out = torch.empty(u.shape[0], C, dtype=u.dtype, device=u.device)
     w, b = weight.float(), bias.float()
