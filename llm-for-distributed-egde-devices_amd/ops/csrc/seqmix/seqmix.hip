@@ -139,7 +139,7 @@ __global__ void __launch_bounds__(NT) gated_norm_kernel(const float* __restrict_
 
 // ---------------------------------------------------------------------------------- rotary + paged write
 // proj row = q [H, D] | k [G, D] | v [G, Dv]; cs [positions, rot / 2, 2]
-template <typename T>
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) rope_write_kernel(const T* __restrict__ proj, int ld, const int* __restrict__ tok_seq,
                                                         const int* __restrict__ tok_pos, const int* __restrict__ seq_slot,
                                                         const int* __restrict__ ptab, int ptab_ld,
@@ -152,6 +152,31 @@ __global__ void __launch_bounds__(NT) rope_write_kernel(const T* __restrict__ pr
   const T* row = proj + (size_t)t * ld;
   const int half = rot >> 1, nqk = (H + G) * D;
   const float* c = cs ? cs + (size_t)pos * rot : nullptr;          // rot / 2 pairs of (cos, sin)
+  if constexpr (VEC) {                                       // 8 coordinates per thread (D, Dv, rot / 2, ld: multiples of 8)
+    for (int e = threadIdx.x * 8; e < nqk; e += NT * 8) {
+      const int hh = e / D, d = e % D;
+      float v[8];
+      load8<T>(row + e, v);
+      if (d < rot) {
+        const int i = d < half ? d : d - half;
+        float o[8], tab[16];
+        load8<T>(row + (d < half ? e + half : e - half), o);
+        load8<float>(c + 2 * i, tab);
+        load8<float>(c + 2 * i + 8, tab + 8);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          v[k] = d < half ? v[k] * tab[2 * k] - o[k] * tab[2 * k + 1] : v[k] * tab[2 * k] + o[k] * tab[2 * k + 1];
+      }
+      if (hh < H) store8<T>(q_out + (size_t)t * H * D + e, v);
+      else store8<T>(kp + (prow * G + (hh - H)) * D + d, v);
+    }
+    for (int e = threadIdx.x * 8; e < G * Dv; e += NT * 8)
+      *reinterpret_cast<uint4*>(vp + prow * G * Dv + e) = *reinterpret_cast<const uint4*>(row + nqk + e);
+    if constexpr (sizeof(T) == 4)                            // fp32 rows: the second 16 bytes of each chunk
+      for (int e = threadIdx.x * 8; e < G * Dv; e += NT * 8)
+        *reinterpret_cast<uint4*>(vp + prow * G * Dv + e + 4) = *reinterpret_cast<const uint4*>(row + nqk + e + 4);
+    return;
+  }
   for (int e = threadIdx.x; e < nqk; e += NT) {
     const int hh = e / D, d = e % D;
     float v = ldf<T>(row + e);
@@ -473,6 +498,8 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
   __shared__ __attribute__((aligned(16))) char k_lds[MK * KS];
   __shared__ __attribute__((aligned(16))) char v_lds[MK * VS];
   __shared__ __attribute__((aligned(16))) char p_all[4 * 16 * PS];
+  constexpr int NPID = 1024;
+  __shared__ int pid_s[NPID];                                // the sequence's first page ids (one global hop per tile less)
   typedef __attribute__((address_space(3))) v4s lds_v4s;
   int qt = blockIdx.x, s = 0;
   for (; s < n; ++s) {
@@ -505,6 +532,9 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
   const int jlo = window > 0 ? max(0, imin - window + 1) : 0;
   const int nbmax = (window > 0 && pool > 0 && imax - window + 1 > 0) ? (imax - window + 1) / pool : 0;
   const int tok_tiles = imax / MK - jlo / MK + 1, ntiles = tok_tiles + (nbmax + MK - 1) / MK;
+  for (int i = tid; i < min(imax / MK + 1, NPID); i += NT) pid_s[i] = pt[i];
+  __syncthreads();
+  auto page_of = [&](int idx) { return idx < NPID ? pid_s[idx] : pt[idx]; };
 
   // a tile's rows travel global -> registers while the tile before it computes, registers -> LDS
   // between the two barriers
@@ -514,7 +544,7 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
   auto load_tile = [&](int tile) {
     const bool tok = tile < tok_tiles;
     const int base = tok ? (jlo / MK + tile) * MK : (tile - tok_tiles) * MK;
-    const size_t prow = tok ? (size_t)pt[base / MK] * MK : 0;
+    const size_t prow = tok ? (size_t)page_of(base / MK) * MK : 0;
 #pragma unroll
     for (int i = 0; i < KL + VL; ++i) {
       const bool isk = i < KL;
@@ -526,7 +556,7 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
                 : *reinterpret_cast<const uint4*>(vp + ((prow + r) * G + g) * Dv + c * 8);
       } else if (base + r < nbmax) {
         const int p0 = (base + r) * pool;
-        const size_t row = ((size_t)pt[p0 / MK] * PB + (p0 % MK) / pool) * G + g;
+        const size_t row = ((size_t)page_of(p0 / MK) * PB + (p0 % MK) / pool) * G + g;
         float f[8];
         load8<float>(isk ? kb + row * D + c * 8 : vb + row * Dv + c * 8, f);
         v = pack8(f);
@@ -1045,8 +1075,12 @@ int edge_sm_rope_write(const void* proj, int ld, const int* tok_seq, const int* 
                        int H, int G, int D, int Dv, int rot, int page, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   if (rot % 2 || rot > D || (rot > 0 && !cs)) return -2;
-  SM_T(f32, hipLaunchKernelGGL(rope_write_kernel<T>, dim3(rows), dim3(NT), 0, st, (const T*)proj, ld, tok_seq, tok_pos,
-                               seq_slot, ptab, ptab_ld, cs, (T*)q_out, (T*)kp, (T*)vp, H, G, D, Dv, rot, page));
+  if (D % 8 == 0 && Dv % 8 == 0 && rot % 16 == 0 && ld % 8 == 0 && ((uintptr_t)proj & 31) == 0)
+    SM_T(f32, hipLaunchKernelGGL((rope_write_kernel<T, true>), dim3(rows), dim3(NT), 0, st, (const T*)proj, ld, tok_seq,
+                                 tok_pos, seq_slot, ptab, ptab_ld, cs, (T*)q_out, (T*)kp, (T*)vp, H, G, D, Dv, rot, page));
+  else
+    SM_T(f32, hipLaunchKernelGGL((rope_write_kernel<T, false>), dim3(rows), dim3(NT), 0, st, (const T*)proj, ld, tok_seq,
+                                 tok_pos, seq_slot, ptab, ptab_ld, cs, (T*)q_out, (T*)kp, (T*)vp, H, G, D, Dv, rot, page));
   return (int)hipGetLastError();
 }
 
