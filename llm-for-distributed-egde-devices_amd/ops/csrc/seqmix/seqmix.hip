@@ -668,62 +668,79 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
 // ---------------------------------------------------------------------------------- convolution
 constexpr int MAX_TAPS = 16;
 
+constexpr int TOKB = 16;                                     // tokens per workgroup on prompt-sized steps: weights are read once for all of them
+
 template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) conv_kernel(const T* __restrict__ u, int ld, int c0, int C,
                                                   const float* __restrict__ w, const float* __restrict__ bias,
                                                   const T* state, const int* __restrict__ tok_seq,
                                                   const int* __restrict__ tok_pos, const int* __restrict__ seq_slot,
                                                   const int* __restrict__ seq_start, const int* __restrict__ seq_off,
-                                                  T* __restrict__ out, int taps, T* state_w) {
+                                                  T* __restrict__ out, int taps, T* state_w, int rows, int tokb) {
   // state_w (steps in which every sequence brings one token: the thread of (token, channel) is the only
   // reader of that channel's tail): the tail is shifted here and no second launch follows
-  const int t = blockIdx.x, s = tok_seq[t];
-  const int pos = tok_pos[t], start = seq_start[s], off = seq_off[s];
-  const T* st = state + (size_t)seq_slot[s] * (taps - 1) * C;
-  T* stw = state_w ? state_w + (size_t)seq_slot[s] * (taps - 1) * C : nullptr;
+  const int t0 = blockIdx.x * tokb, t1 = min(rows, t0 + tokb);
   if constexpr (VEC) {                                       // eight channels per thread (ld, c0, C multiples of 8)
     for (int c = (blockIdx.y * NT + threadIdx.x) * 8; c < C; c += NT * gridDim.y * 8) {
-      float acc[8];
+      float br[8], wr[8][4];                                 // up to four taps stay in registers
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = bias[c + e];
-      for (int k0 = 0; k0 < taps; k0 += 4) {                 // four taps' rows in flight
-        float x[4][8];
+      for (int e = 0; e < 8; ++e) {
+        br[e] = bias[c + e];
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          const int k = k0 + kk, p = pos - (taps - 1) + k;
-          if (k < taps && p >= start) load8<T>(u + (size_t)(off + p - start) * ld + c0 + c, x[kk]);
-          else if (k < taps && p >= 0) load8<T>(st + (size_t)(p - (start - (taps - 1))) * C + c, x[kk]);
-          else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[kk][e] = 0.f;
-          }
-        }
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          if (k0 + kk < taps) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] += w[(c + e) * taps + k0 + kk] * x[kk][e];
-            // the new tail = inputs of positions pos - (taps - 2) .. pos = taps 1 .. taps - 1 of this window
-            if (stw && k0 + kk >= 1) store8<T>(stw + (size_t)(k0 + kk - 1) * C + c, x[kk]);
-          }
-        }
+        for (int k = 0; k < 4; ++k) wr[e][k] = k < taps ? w[(c + e) * taps + k] : 0.f;
       }
+      for (int t = t0; t < t1; ++t) {
+        const int s = tok_seq[t], pos = tok_pos[t], start = seq_start[s], off = seq_off[s];
+        const T* st = state + (size_t)seq_slot[s] * (taps - 1) * C;
+        T* stw = state_w ? state_w + (size_t)seq_slot[s] * (taps - 1) * C : nullptr;
+        float acc[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
-      store8<T>(out + (size_t)t * C + c, acc);
+        for (int e = 0; e < 8; ++e) acc[e] = br[e];
+        for (int k0 = 0; k0 < taps; k0 += 4) {               // four taps' rows in flight
+          float x[4][8];
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk) {
+            const int k = k0 + kk, p = pos - (taps - 1) + k;
+            if (k < taps && p >= start) load8<T>(u + (size_t)(off + p - start) * ld + c0 + c, x[kk]);
+            else if (k < taps && p >= 0) load8<T>(st + (size_t)(p - (start - (taps - 1))) * C + c, x[kk]);
+            else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) x[kk][e] = 0.f;
+            }
+          }
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk) {
+            if (k0 + kk < taps) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                acc[e] += (k0 == 0 ? wr[e][kk] : w[(c + e) * taps + k0 + kk]) * x[kk][e];
+              // the new tail = inputs of positions pos - (taps - 2) .. pos = taps 1 .. taps - 1 of this window
+              if (stw && k0 + kk >= 1) store8<T>(stw + (size_t)(k0 + kk - 1) * C + c, x[kk]);
+            }
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = siluf_(acc[e]);
+        store8<T>(out + (size_t)t * C + c, acc);
+      }
     }
   } else {
-    for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
-      float acc = bias[c];
-      for (int k = 0; k < taps; ++k) {
-        const int p = pos - (taps - 1) + k;
-        float x = 0.f;
-        if (p >= start) x = ldf<T>(u + (size_t)(off + p - start) * ld + c0 + c);
-        else if (p >= 0) x = ldf<T>(st + (size_t)(p - (start - (taps - 1))) * C + c);
-        acc += w[c * taps + k] * x;
-        if (stw && k >= 1) stf<T>(stw + (size_t)(k - 1) * C + c, x);
+    for (int t = t0; t < t1; ++t) {
+      const int s = tok_seq[t], pos = tok_pos[t], start = seq_start[s], off = seq_off[s];
+      const T* st = state + (size_t)seq_slot[s] * (taps - 1) * C;
+      T* stw = state_w ? state_w + (size_t)seq_slot[s] * (taps - 1) * C : nullptr;
+      for (int c = blockIdx.y * NT + threadIdx.x; c < C; c += NT * gridDim.y) {
+        float acc = bias[c];
+        for (int k = 0; k < taps; ++k) {
+          const int p = pos - (taps - 1) + k;
+          float x = 0.f;
+          if (p >= start) x = ldf<T>(u + (size_t)(off + p - start) * ld + c0 + c);
+          else if (p >= 0) x = ldf<T>(st + (size_t)(p - (start - (taps - 1))) * C + c);
+          acc += w[c * taps + k] * x;
+          if (stw && k >= 1) stf<T>(stw + (size_t)(k - 1) * C + c, x);
+        }
+        stf<T>(out + (size_t)t * C + c, siluf_(acc));
       }
-      stf<T>(out + (size_t)t * C + c, siluf_(acc));
     }
   }
 }
@@ -778,6 +795,27 @@ __global__ void __launch_bounds__(64) ssd_kernel(const T* __restrict__ xbc, int 
 #pragma unroll
   for (int n = 0; n < NMAX; ++n) S[n] = (start > 0 && n < N && p < P) ? st[(size_t)n * P + p] : 0.f;
   const float a = expf(A_log[h]), Dh = Dp[h], bias = dt_bias[h];
+  if (len == 1) {
+    // one token (decode): no staging; B, C, x, the step size and the state rows are independent loads
+    if (p < P) {
+      const size_t row = (size_t)off;
+      const float raw = ldf<T>(u + row * ld + dt0 + h) + bias;
+      const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+      const float dec = expf(-a * dt), xv = ldf<T>(xbc + row * Cx + h * P + p), dx = dt * xv;
+      const T* bc = xbc + row * Cx + inner + g * N;
+      float yv = 0.f;
+#pragma unroll
+      for (int n = 0; n < NMAX; ++n) {
+        if (n < N) {
+          const float Sn = dec * S[n] + ldf<T>(bc + n) * dx;
+          yv += Sn * ldf<T>(bc + groups * N + n);
+          st[(size_t)n * P + p] = Sn;
+        }
+      }
+      y[row * inner + h * P + p] = yv + Dh * xv;
+    }
+    return;
+  }
   for (int t0 = 0; t0 < len; t0 += TC) {
     const int tc = min(TC, len - t0);
     __syncthreads();
@@ -1150,15 +1188,16 @@ int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, cons
   if (rows == 0) return 0;
   if (taps < 1 || taps > MAX_TAPS) return -2;
   const bool one = max_len == 1 && taps > 1;                 // every sequence brings one token
+  const int tokb = rows >= 64 * TOKB ? TOKB : 1;             // decode-sized steps: one token per workgroup
   const int gy = (C + NT - 1) / NT;
   if (ld % 8 == 0 && c0 % 8 == 0 && C % 8 == 0)
-    SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, true>), dim3(rows, (C / 8 + NT - 1) / NT), dim3(NT), 0, st,
-                                 (const T*)u, ld, c0, C, w, bias, (const T*)state, tok_seq, tok_pos, seq_slot,
-                                 seq_start, seq_off, (T*)out, taps, one ? (T*)state : (T*)nullptr));
+    SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, true>), dim3((rows + tokb - 1) / tokb, (C / 8 + NT - 1) / NT), dim3(NT),
+                                 0, st, (const T*)u, ld, c0, C, w, bias, (const T*)state, tok_seq, tok_pos, seq_slot,
+                                 seq_start, seq_off, (T*)out, taps, one ? (T*)state : (T*)nullptr, rows, tokb));
   else
-    SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, false>), dim3(rows, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, w,
-                                 bias, (const T*)state, tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps,
-                                 one ? (T*)state : (T*)nullptr));
+    SM_T(f32, hipLaunchKernelGGL((conv_kernel<T, false>), dim3((rows + tokb - 1) / tokb, gy), dim3(NT), 0, st,
+                                 (const T*)u, ld, c0, C, w, bias, (const T*)state, tok_seq, tok_pos, seq_slot, seq_start,
+                                 seq_off, (T*)out, taps, one ? (T*)state : (T*)nullptr, rows, tokb));
   if (taps > 1 && !one)
     SM_T(f32, hipLaunchKernelGGL(conv_state_kernel<T>, dim3(n, gy), dim3(NT), 0, st, (const T*)u, ld, c0, C, (T*)state,
                                  seq_slot, seq_start, seq_len, seq_off, taps));

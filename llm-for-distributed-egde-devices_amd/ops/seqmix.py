@@ -305,11 +305,12 @@ def conv_silu(u: torch.Tensor, c0: int, C: int, weight: torch.Tensor, bias: torc
     w, b = weight.float(), bias.float()
     for slot, start, n, off in meta.host:
         x = u[off:off + n, c0:c0 + C].float()
-        hist = state[slot].float() if start > 0 else torch.zeros(taps - 1, C, device=u.device)
+        hist = state[slot, :taps - 1].float() if start > 0 else torch.zeros(taps - 1, C, device=u.device)
         xin = torch.cat([hist, x], 0)                             # [taps - 1 + n, C]
         win = xin.unfold(0, taps, 1)                              # [n, C, taps]
         out[off:off + n] = F.silu((win * w[None]).sum(-1) + b).to(u.dtype)
-        state[slot] = xin[xin.shape[0] - (taps - 1):].to(state.dtype)
+        if taps > 1:
+            state[slot, :taps - 1] = xin[xin.shape[0] - (taps - 1):].to(state.dtype)
     return out
 
 

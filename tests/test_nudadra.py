@@ -203,7 +203,8 @@ def test_attention_op_portions_and_a_far_key(dev, window, pool, H, G, D, Dv, pag
 @pytest.mark.parametrize("Hs,P,N,groups,taps,sizes", [
     (2, 4, 3, 1, 4, (1, 2, 3, 4, 5)), (4, 8, 16, 2, 2, (1, 2, 3, 4, 5)), (3, 5, 20, 3, 5, (1, 2, 3, 4, 5)),
     (1, 70, 33, 1, 3, (1, 2, 3, 4, 5)), (2, 70, 67, 2, 4, (64, 1, 33, 65, 2, 130)), (3, 16, 8, 1, 3, (40, 100, 7)),
-    (8, 8, 8, 1, 4, (1, 2, 3, 4, 5)), (8, 8, 8, 1, 4, (40, 100, 7))])
+    (8, 8, 8, 1, 4, (1, 2, 3, 4, 5)), (8, 8, 8, 1, 4, (40, 100, 7)), (8, 8, 8, 1, 4, (1030, 70, 5)),
+    (3, 5, 20, 3, 5, (1030, 70, 5))])
 def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps, sizes):
     """Convolution tail and state matrix carried over portions of ``sizes`` tokens (short ones step
     token by token, long ones take the chunked form; chunk borders inside and at the end of a
@@ -211,7 +212,7 @@ def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps, sizes):
     whole sequence."""
     torch.manual_seed(2)
     inner, C = Hs * P, Hs * P + 2 * groups * N
-    Ts = {0: 23, 2: 17} if max(sizes) < 10 else {0: 300, 2: 171}
+    Ts = {0: 23, 2: 17} if max(sizes) < 10 else ({0: 300, 2: 171} if max(sizes) < 1000 else {0: 1105, 2: 171})
     u = {s: torch.randn(T, 2 * inner + 2 * groups * N + Hs, dtype=torch.float64) for s, T in Ts.items()}
     cw, cb = torch.randn(C, taps, dtype=torch.float64) * 0.5, torch.randn(C, dtype=torch.float64) * 0.2
     dtb, A_log, Dp = torch.randn(Hs, dtype=torch.float64), torch.rand(Hs, dtype=torch.float64) - 0.5, torch.randn(Hs, dtype=torch.float64)
@@ -243,7 +244,10 @@ def test_state_space_ops_in_portions(dev, Hs, P, N, groups, taps, sizes):
             off += m
             at[s] += m
     for s in Ts:
-        assert torch.allclose(torch.cat(got[s]), want[s], atol=3e-5, rtol=1e-4), s
+        g = torch.cat(got[s])
+        # fp32 sums regrouped per 64-token chunk against float64: the error grows with the state's size
+        err = ((g - want[s]).abs() / (1.0 + want[s].abs())).max().item()
+        assert err < (3e-5 if max(sizes) < 1000 else 1e-4), (s, err)
 
 
 @pytest.mark.parametrize("dev", DEVS)
@@ -502,3 +506,59 @@ models: ["{d}"]
     out = evaluate.main(["--config", str(y), "--devices", "cpu", "--num_samples", "2", "--max_seq", "256",
                          "--batch_size", "2", "--prefill_chunk", "16", "--precision", "fp32"])
     assert out[str(d)]["tps"] > 0 and 0 < out[str(d)]["confidence"] <= 1
+
+
+def _random_config(seed):
+    import random
+    r = random.Random(seed)
+    kv = r.choice([1, 2, 3])
+    heads = kv * r.choice([1, 2, 4])
+    dim = r.choice([4, 8, 12, 16, 32])
+    s_heads = r.choice([1, 2, 4])
+    groups = r.choice([g for g in (1, 2, 4) if s_heads % g == 0])
+    s_vdim = r.choice([4, 8, 12])
+    n_layers = r.choice([1, 2, 3])
+    loop = None
+    if r.random() < 0.6:
+        a = r.randrange(0, n_layers)
+        loop = (a, r.randrange(a + 1, n_layers + 1), r.choice([1, 2, 3]))
+    return make_config(width=r.choice([24, 40, 64]), vocab=r.choice([37, 64, 101]), n_layers=n_layers, heads=heads,
+                       kv_heads=kv, dim=dim, vdim=r.choice([dim, 8, 20]), window=r.choice([3, 5, 16, 33, None]),
+                       pool=r.choice([1, 2, 5, 8]), rot_dims=r.choice([0, dim, dim // 2]), scaling=r.random() < 0.5,
+                       s_heads=s_heads, s_vdim=s_vdim, state=r.choice([1, 4, 7, 16]), groups=groups,
+                       conv=r.choice([1, 2, 3, 4, 6]), norm_groups=r.choice([g for g in (1, 2, 4) if (s_heads * s_vdim) % g == 0]),
+                       ff=r.choice([None, 16, 56]), loop=loop)
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("seed", range(8))
+def test_random_geometries(tmp_path, dev, seed):
+    """Sizes drawn at random (head counts and ratios, key / value sizes, windows, pools, rotation
+    share, state sizes, taps, norm groups, loops, missing feed-forward): a prompt in portions with
+    token-by-token decoding and a second request beside it, against the oracle."""
+    cfg = _random_config(100 + seed)
+    w = make_weights(cfg, seed=seed)
+    model = load(tmp_path, cfg, w, dev)
+    reqs = {"a": tokens(50, cfg["vocab"], seed), "b": tokens(21, cfg["vocab"], seed + 50)}
+    want = {r: oracle.forward(cfg, w, t) for r, t in reqs.items()}
+    sched = [[("a", 17)], [("a", 2), ("b", 20)], [("a", 18), ("b", 1)]] + [[("a", 1)]] * 13
+    got, _ = replay(model, sched, reqs, 128, slots=2)
+    for r in reqs:
+        assert close(got[r], want[r], TOL["fp32"]), (r, cfg)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim,heads,kv", [(32, 2, 1), (64, 4, 2)])
+def test_bf16_model_on_the_matrix_core_prompt_kernel(tmp_path, dim, heads, kv):
+    """A bf16 model whose head sizes the matrix-core prompt kernel takes: prompts in portions of 16+
+    tokens (that kernel) and decoded tokens (the general kernel) agree with the oracle within rounding."""
+    cfg = make_config(width=64, n_layers=2, loop=(1, 2, 2), heads=heads, kv_heads=kv, dim=dim, vdim=dim, rot_dims=dim,
+                      window=48, pool=8, s_heads=2, s_vdim=16, state=8, ff=64)
+    w = make_weights(cfg, seed=31)
+    model = load(tmp_path, cfg, w, "cuda", precision="bf16")
+    reqs = {"a": tokens(200, cfg["vocab"], 1), "b": tokens(90, cfg["vocab"], 2)}
+    want = {r: oracle.forward(cfg, w, t) for r, t in reqs.items()}
+    sched = [[("a", 70), ("b", 33)], [("a", 64), ("b", 1)], [("a", 50), ("b", 40)]] + [[("a", 1), ("b", 1)]] * 16
+    got, _ = replay(model, sched, reqs, 512, slots=2)
+    for r in reqs:
+        assert close(got[r], want[r], TOL["bf16"]), r
