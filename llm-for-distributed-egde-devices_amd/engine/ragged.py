@@ -72,8 +72,15 @@ class _DecodeGraph:
         if self.graph is None:
             g = torch.cuda.CUDAGraph()
             torch.cuda.synchronize()
-            with torch.cuda.graph(g, pool=eng._pool):
-                self.out = eng.model(self.ids, self.meta, eng.cache, self.rows)
+            try:
+                with torch.cuda.graph(g, pool=eng._pool):
+                    self.out = eng.model(self.ids, self.meta, eng.cache, self.rows)
+            except Exception as e:  # noqa: BLE001 - an op that cannot be captured: this engine steps eagerly
+                from ..utils.log import get_logger
+                get_logger("ragged").warning(f"decode step not graph-capturable ({e!r}): running eagerly")
+                torch.cuda.synchronize()
+                eng.use_graphs = False
+                return eng.model(self.ids, self.meta, eng.cache, self.rows)
             if eng._pool is None:
                 eng._pool = g.pool()
             self.graph = g

@@ -486,7 +486,8 @@ __global__ void __launch_bounds__(NT) attn_merge_kernel(const float* __restrict_
 // row-major V tile.  Tiles wholly outside a workgroup's window are never visited.
 constexpr int MQ = 64, MK = 64;
 
-template <int DK, int DV>
+// RH query heads of one kv head per workgroup: a staged key / value tile serves all of them
+template <int DK, int DV, int RH>
 __global__ void __launch_bounds__(NT) attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ gate, int gate_ld, const bf16_t* __restrict__ kp,
     const bf16_t* __restrict__ vp, const float* __restrict__ kb, const float* __restrict__ vb,
@@ -508,26 +509,31 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
     qt -= nq;
   }
   if (s == n) return;
-  const int h = blockIdx.y, g = h / (H / G);
+  const int h0 = blockIdx.y * RH, g = h0 / (H / G);
   const int start = seq_start[s], len = seq_len[s], off = seq_off[s];
   const int* pt = ptab + (size_t)seq_slot[s] * ptab_ld;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, c16 = lane & 15;
   char* p_lds = p_all + wave * 16 * PS;
   const int wq0 = qt * MQ + wave * 16;                       // this wave's first row inside the portion
-  v8s qf[DK];
+  v8s qf[RH][DK];
   {
     const int t = wq0 + c16;
 #pragma unroll
-    for (int kk = 0; kk < DK; ++kk)
-      qf[kk] = t < len ? *reinterpret_cast<const v8s*>(q + ((size_t)(off + t) * H + h) * D + kk * 32 + 8 * g4)
-                       : v8s{0, 0, 0, 0, 0, 0, 0, 0};
+    for (int r = 0; r < RH; ++r)
+#pragma unroll
+      for (int kk = 0; kk < DK; ++kk)
+        qf[r][kk] = t < len ? *reinterpret_cast<const v8s*>(q + ((size_t)(off + t) * H + h0 + r) * D + kk * 32 + 8 * g4)
+                            : v8s{0, 0, 0, 0, 0, 0, 0, 0};
   }
-  v4f o[DV];
+  v4f o[RH][DV];
+  float m_i[RH][4], l_i[RH][4];
 #pragma unroll
-  for (int i = 0; i < DV; ++i) o[i] = v4f{0.f, 0.f, 0.f, 0.f};
-  float m_i[4], l_i[4];
+  for (int r = 0; r < RH; ++r) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { m_i[i] = -INFINITY; l_i[i] = 0.f; }
+    for (int i = 0; i < DV; ++i) o[r][i] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { m_i[r][i] = -INFINITY; l_i[r][i] = 0.f; }
+  }
   const int imin = start + qt * MQ, imax = start + min(len, qt * MQ + MQ) - 1;
   const int jlo = window > 0 ? max(0, imin - window + 1) : 0;
   const int nbmax = (window > 0 && pool > 0 && imax - window + 1 > 0) ? (imax - window + 1) / pool : 0;
@@ -585,6 +591,8 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
     store_tile();
     __syncthreads();
     if (tile + 1 < ntiles) load_tile(tile + 1);
+#pragma unroll
+    for (int r = 0; r < RH; ++r) {
     v4f sc[4];
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
@@ -592,7 +600,7 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
 #pragma unroll
       for (int kk = 0; kk < DK; ++kk) {
         const v8s kf = *reinterpret_cast<const v8s*>(k_lds + (nt * 16 + c16) * KS + (kk * 32 + 8 * g4) * 2);
-        sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], kf, sc[nt], 0, 0, 0);
+        sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[r][kk], kf, sc[nt], 0, 0, 0);
       }
     }
     // lane holds S[row = 4 g4 + i][key = 16 nt + c16]
@@ -612,9 +620,9 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
       }
 #pragma unroll
       for (int o_ = 1; o_ < 16; o_ <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o_, 64));
-      const float mnew = fmaxf(m_i[i], mx);
+      const float mnew = fmaxf(m_i[r][i], mx);
       const float msafe = (mnew == -INFINITY) ? 0.f : mnew;
-      alpha[i] = __builtin_amdgcn_exp2f(m_i[i] - msafe);
+      alpha[i] = __builtin_amdgcn_exp2f(m_i[r][i] - msafe);
       float rs = 0.f;
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
@@ -624,13 +632,13 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
       }
 #pragma unroll
       for (int o_ = 1; o_ < 16; o_ <<= 1) rs += __shfl_xor(rs, o_, 64);
-      l_i[i] = l_i[i] * alpha[i] + rs;
-      m_i[i] = mnew;
+      l_i[r][i] = l_i[r][i] * alpha[i] + rs;
+      m_i[r][i] = mnew;
     }
 #pragma unroll
     for (int dt = 0; dt < DV; ++dt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[dt][i] *= alpha[i];
+      for (int i = 0; i < 4; ++i) o[r][dt][i] *= alpha[i];
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
@@ -648,19 +656,24 @@ __global__ void __launch_bounds__(NT) attn_mfma_kernel(
         const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(a0));
         const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s*)(a0 + 4 * VS));
         const v8s vf = v8s{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[dt], 0, 0, 0);
+        o[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[r][dt], 0, 0, 0);
       }
+    }
+      __builtin_amdgcn_wave_barrier();                     // this wave's P reads precede the next head's P writes
     }
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int t = wq0 + 4 * g4 + i;
     if (t < len) {
-      float inv = l_i[i] > 0.f ? 1.f / l_i[i] : 0.f;
-      if (gate) inv *= sigmoidf_(bf2f(gate[(size_t)(off + t) * gate_ld + h]));
 #pragma unroll
-      for (int dt = 0; dt < DV; ++dt)
-        out[((size_t)(off + t) * H + h) * Dv + dt * 16 + c16] = f2bf(o[dt][i] * inv);
+      for (int r = 0; r < RH; ++r) {
+        float inv = l_i[r][i] > 0.f ? 1.f / l_i[r][i] : 0.f;
+        if (gate) inv *= sigmoidf_(bf2f(gate[(size_t)(off + t) * gate_ld + h0 + r]));
+#pragma unroll
+        for (int dt = 0; dt < DV; ++dt)
+          out[((size_t)(off + t) * H + h0 + r) * Dv + dt * 16 + c16] = f2bf(o[r][dt][i] * inv);
+      }
     }
   }
 }
@@ -1252,10 +1265,24 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
   if (page != MK || G <= 0 || H % G) return 1;
   if (n == 0 || qtiles == 0) return 0;
   const float sl2 = scale * 1.4426950408889634f;
-#define SM_MF(DK, DV)                                                                                              \
-  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV>), dim3(qtiles, H), dim3(NT), 0, st, (const bf16_t*)q,              \
+  // query heads per workgroup: a staged tile can serve 4 or 2 heads of a kv group, but the kernel is
+  // bound by each wave's MFMA -> softmax -> LDS -> MFMA chain and needs ~4 waves per SIMD to hide it
+  // (4096-token prompt, 16 heads: 111 us with one head per workgroup, 190 us with four), so heads are
+  // grouped only while >= 1024 workgroups remain
+  const int R = H / G;
+  int rh = 1;
+  if (R % 4 == 0 && (long)qtiles * (H / 4) >= 1024) rh = 4;
+  else if (R % 2 == 0 && (long)qtiles * (H / 2) >= 1024) rh = 2;
+#define SM_MF_R(DK, DV, RH)                                                                                        \
+  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV, RH>), dim3(qtiles, H / RH), dim3(NT), 0, st, (const bf16_t*)q,     \
                      (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb, seq_slot,         \
                      seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window, pool)
+#define SM_MF(DK, DV)                      \
+  do {                                     \
+    if (rh == 4) SM_MF_R(DK, DV, 4);       \
+    else if (rh == 2) SM_MF_R(DK, DV, 2);  \
+    else SM_MF_R(DK, DV, 1);               \
+  } while (0)
   if (D == 64 && Dv == 64) SM_MF(2, 4);
   else if (D == 96 && Dv == 96) SM_MF(3, 6);
   else if (D == 128 && Dv == 128) SM_MF(4, 8);
@@ -1264,6 +1291,7 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
   else if (D == 32 && Dv == 32) SM_MF(1, 2);
   else return 1;
 #undef SM_MF
+#undef SM_MF_R
   return (int)hipGetLastError();
 }
 

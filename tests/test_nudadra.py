@@ -439,7 +439,7 @@ def test_decode_graph_replays_match_eager(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("window,pool,H,G,D,Dv", [(40, 8, 4, 2, 32, 32), (100, 16, 2, 1, 64, 64), (None, None, 2, 2, 32, 32),
-                                                  (70, 3, 3, 1, 96, 96), (33, 70, 2, 2, 128, 64), (300, 2, 4, 2, 32, 32)])
+                                                  (70, 3, 3, 1, 96, 96), (33, 70, 2, 2, 128, 64), (300, 2, 4, 2, 32, 32), (64, 8, 8, 2, 32, 32), (50, 4, 4, 1, 64, 64)])
 def test_attention_bf16_prompt_kernel(window, pool, H, G, D, Dv):
     """The matrix-core prompt kernel (bf16 portions of 16 tokens or more): two sequences in the
     same steps, portions that start and end inside pages, a planted far key, against the oracle on
