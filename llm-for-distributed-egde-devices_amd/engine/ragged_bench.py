@@ -36,7 +36,7 @@ SIZES = {
 
 def hybrid_config(s: dict) -> ModelConfig:
     a = WindowAttnSpec(s["heads"], s["kv"], s["dim"], s["dim"], s["dim"] ** -0.5, s["window"], s["pool"], s["dim"],
-                       500000.0, {"rope_type": "yarn", "factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0})
+                       500000.0, {"rope_type": "yarn", "factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0})
     m = SSDSpec(s["s_heads"], s["s_vdim"], s["state"], 1, 4, 1)
     specs = [LayerSpec("parallel", a, m, s["ff"]) for _ in range(s["layers"])]
     return ModelConfig(arch="nudadra", vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
