@@ -487,8 +487,10 @@ __global__ void __launch_bounds__(NT) attn_merge_kernel(const float* __restrict_
 constexpr int MQ = 64, MK = 64;
 
 // RH query heads of one kv head per workgroup: a staged key / value tile serves all of them
+// (second launch bound: workgroups per CU the register budget must allow - four for 64-wide heads, so the
+// 1024 workgroups of a 4096-token, 16-head prompt are resident at once)
 template <int DK, int DV, int RH>
-__global__ void __launch_bounds__(NT) attn_mfma_kernel(
+__global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1))) attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ gate, int gate_ld, const bf16_t* __restrict__ kp,
     const bf16_t* __restrict__ vp, const float* __restrict__ kb, const float* __restrict__ vb,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_len,
