@@ -562,3 +562,38 @@ def test_bf16_model_on_the_matrix_core_prompt_kernel(tmp_path, dim, heads, kv):
     got, _ = replay(model, sched, reqs, 512, slots=2)
     for r in reqs:
         assert close(got[r], want[r], TOL["bf16"]), r
+
+
+def test_trace_runner_program(tmp_path):
+    """``bin/trace_run`` as a program: steps on standard input, a flushed ``done <step>`` per step,
+    logits files only for steps that want rows (little-endian fp32 [wanted, vocab], entry order),
+    requests ended and their slot reused, exit code 0 at end of input."""
+    import subprocess
+    import numpy as np
+    from safetensors.torch import save_file
+    cfg = make_config(n_layers=2, loop=(1, 2, 2), window=10, pool=4)
+    w = make_weights(cfg, seed=41)
+    d = tmp_path / "m"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file(w, str(d / "model.safetensors"))
+    a, b, c = tokens(30, cfg["vocab"], 1), tokens(9, cfg["vocab"], 2), tokens(12, cfg["vocab"], 3)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:20], "want": [0, 19]}, {"id": "b", "tokens": b, "want": [8]}],
+              "end": ["b"]},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[20:29], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "c", "tokens": c, "want": [11]}, {"id": "a", "tokens": a[29:], "want": [0]}],
+              "end": ["a", "c"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(d), "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128", "--slots", "2", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert sorted(os.listdir(out)) == ["0.f32", "2.f32"]
+    V = cfg["vocab"]
+    wa, wb, wc = (oracle.forward(cfg, w, t) for t in (a, b, c))
+    g0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V))
+    g2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V))
+    assert close(g0, torch.stack([wa[0], wa[19], wb[8]]), TOL["fp32"])
+    assert close(g2, torch.stack([wc[11], wa[29]]), TOL["fp32"])
