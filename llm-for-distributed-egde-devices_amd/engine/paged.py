@@ -12,7 +12,11 @@ Per run:
   k_pool / v_pool [pages, ceil(page / pool), kv heads, D | Dv]  fp32 block means; block b sits
       beside the page of its first token b*pool, at entry (b*pool mod page) // pool
   conv [slots, taps - 1, channels]                              the convolution's last inputs
-  ssm  [slots, heads, N, vdim] fp32                             the state-space matrix
+  ssm  [slots, heads, N, vdim] fp32                             the state-space / delta-rule matrix
+  lat  [pages, page, 1, kv_rank + R]                            latent attention: normed latent | rotated
+      shared key part; a layer that reads another layer's cache holds the same tensor as that run
+  canon1 / canon2 [slots, taps - 1, width] fp32                 last inputs of the sublayers' input convolutions
+and, for models whose embedding looks at the previous token, ``prev_tok`` int64 [slots].
 A slot's recurrent rows are not cleared on release: a portion that starts at position 0 ignores
 what the slot held (the kernels start from zero there).
 """
@@ -24,17 +28,43 @@ import torch
 
 
 class RunCache:
-    __slots__ = ("k", "v", "k_pool", "v_pool", "conv", "ssm")
+    __slots__ = ("k", "v", "k_pool", "v_pool", "conv", "ssm", "lat", "canon1", "canon2")
+
+    def __init__(self):
+        for n in self.__slots__:
+            setattr(self, n, None)
 
 
 class PagedCache:
     def __init__(self, run_specs, num_pages: int, slots: int = 4, page: int = 64, dtype=torch.bfloat16,
-                 device=None):
+                 device=None, width: int = 0, canon_taps: int = 0, prev_token: bool = False, run_layers=None):
+        """``run_layers``: the layer index of every run (a latent-attention layer's ``kv_from`` names a
+        layer; its cache is the run of that layer)."""
         self.page, self.num_pages, self.slots = page, num_pages, slots
         self.dtype, self.device = dtype, device
         self.runs: List[RunCache] = []
-        for s in run_specs:
+        self.prev_tok = torch.zeros(slots, dtype=torch.long, device=device) if prev_token else None
+        run_layers = list(run_layers) if run_layers is not None else list(range(len(run_specs)))
+        for r, s in enumerate(run_specs):
             rc = RunCache()
+            latent, delta = getattr(s, "latent", None), getattr(s, "delta", None)
+            if latent is not None or delta is not None:
+                if latent is not None:
+                    src = s.latent.kv_from
+                    if src is None:
+                        rc.lat = torch.zeros(num_pages, page, 1, s.latent.cache_dim, dtype=dtype, device=device)
+                    else:                                  # the latest earlier run of the named layer
+                        rc.lat = self.runs[max(j for j in range(r) if run_layers[j] == src)].lat
+                else:
+                    d = s.delta
+                    rc.conv = torch.zeros(slots, max(d.conv - 1, 1), d.conv_channels, dtype=dtype, device=device)
+                    rc.ssm = torch.zeros(slots, d.heads, d.dim, d.vdim, dtype=torch.float32, device=device)
+                if canon_taps:
+                    rc.canon1 = torch.zeros(slots, max(canon_taps - 1, 1), width, dtype=torch.float32, device=device)
+                    if getattr(s, "moe", None) is not None or getattr(s, "ff", None):
+                        rc.canon2 = torch.zeros_like(rc.canon1)
+                self.runs.append(rc)
+                continue
             a, m = s.attn, s.ssd
             rc.k = torch.zeros(num_pages, page, a.kv_heads, a.dim, dtype=dtype, device=device)
             rc.v = torch.zeros(num_pages, page, a.kv_heads, a.vdim, dtype=dtype, device=device)
@@ -91,11 +121,12 @@ class PagedCache:
         self.free_slots.append(slot)
 
     def nbytes(self) -> int:
-        n = self.page_table.numel() * 4
+        n, seen = self.page_table.numel() * 4, set()
         for rc in self.runs:
             for name in RunCache.__slots__:
                 t = getattr(rc, name)
-                if t is not None:
+                if t is not None and t.data_ptr() not in seen:     # a shared latent cache counts once
+                    seen.add(t.data_ptr())
                     n += t.numel() * t.element_size()
         return n
 

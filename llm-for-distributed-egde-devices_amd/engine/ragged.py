@@ -94,7 +94,10 @@ class RaggedEngine:
         self.model, self.cfg, self.device = model, model.cfg, model.device
         self.page = page
         pages = max(1, (int(max_tokens) + page - 1) // page)
-        self.cache = PagedCache(model.run_specs(), pages, slots, page, dtype=model.dtype, device=self.device)
+        cfg = model.cfg
+        self.cache = PagedCache(model.run_specs(), pages, slots, page, dtype=model.dtype, device=self.device,
+                                width=cfg.hidden_size, canon_taps=cfg.canon_taps, prev_token=bool(cfg.bigram),
+                                run_layers=[i for i, _ in model.runs])
         self.live: Dict[object, int] = {}
         # decode-only steps (every sequence brings one token) replay a HIP graph per batch size
         self.use_graphs = (self.device.type == "cuda" and ops.gpu_path(model.embed)) if use_graphs is None \

@@ -10,6 +10,9 @@ Families (dims are public HF configs):
   * GPT-2                — learned positions, gelu_new (CPU gRPC plumbing config, BASELINE.json)
   * BERT (MiniLM-L6)     — bidirectional encoder used as the sentence embedder
                            (combine_model_fp_updated.py:70-73,179)
+  * layer-spec layouts   — per-layer descriptions (``layer_specs``): Nudadra (windowed attention with
+                           pooled blocks beside a Mamba-2 mixer) and Pagonex (latent attention and
+                           gated delta-rule layers with mixture-of-experts feed-forwards)
 A single ``ModelConfig`` describes all decoder families; ``DecoderLM`` interprets the flags.
 """
 from __future__ import annotations
@@ -73,14 +76,85 @@ class SSDSpec:
 
 
 @dataclass
+class LatentAttnSpec:
+    """Softmax attention through low-rank latents: queries W_uq rms(W_dq h) laid out per head as
+    ``dim`` unrotated | ``rot_dim`` rotated coordinates; keys and values are expanded per head from
+    one cached latent of ``kv_rank`` numbers (W_uk c, W_uv c) plus one rotated key part of
+    ``rot_dim`` numbers shared by all heads.  ``window``: sliding window (None: causal);
+    ``kv_from``: the layer whose cached latent and rotated key part this layer reads instead of
+    projecting its own.  Rotation pairs neighbouring coordinates (2i, 2i + 1)."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    window: Optional[int] = None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional[dict] = None
+    kv_from: Optional[int] = None
+
+    @property
+    def cache_dim(self) -> int:
+        """Numbers cached per token: the latent and the shared rotated key part."""
+        return self.kv_rank + self.rot_dim
+
+
+@dataclass
+class DeltaSpec:
+    """Gated delta rule with one decay per head and key channel: a [dim, vdim] fp32 state per head,
+    q / k shared by ``heads / kv_heads`` heads, a causal depthwise convolution of ``conv`` taps + silu
+    over q | k | v, unit-length q and k, low-rank decay (``decay_rank``) and output-gate
+    (``gate_rank``) projections, an RMS norm per head with one weight vector shared by the heads."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    decay_rank: int
+    gate_rank: int
+
+    @property
+    def conv_channels(self) -> int:
+        return 2 * self.kv_heads * self.dim + self.heads * self.vdim
+
+    @property
+    def in_sizes(self):
+        """Row blocks of the fused input projection: q | k | v | beta | decay down | gate down."""
+        return (self.kv_heads * self.dim, self.kv_heads * self.dim, self.heads * self.vdim, self.heads,
+                self.decay_rank, self.gate_rank)
+
+
+@dataclass
+class MoESpec:
+    """Mixture of clamped gated-linear experts: softmax router over ``experts``, the ``top`` largest
+    renormalised and multiplied by ``scale``; an optional shared expert of width ``shared_ff`` runs
+    for every token.  Expert: g = min(W_g h, limit), u = clamp(W_u h, +-limit),
+    W_d (g sigmoid(1.702 g) (u + 1))."""
+    experts: int
+    top: int
+    scale: float
+    ff: int
+    limit: float
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+
+
+@dataclass
 class LayerSpec:
     """One layer of a ``layer_specs`` model: the mixer kind with its branches, and the feed-forward
-    width (None: the layer has no feed-forward)."""
-    mixer: str                               # "parallel": attention and state-space side by side
+    (``ff``: dense width, ``moe``: mixture of experts; neither: the layer has no feed-forward)."""
+    mixer: str                               # "parallel": attention and state-space side by side;
+                                             # "latent_attention" / "channel_delta": one mixer, norm on the sublayer's output
     attn: Optional[WindowAttnSpec] = None
     ssd: Optional[SSDSpec] = None
     ff: Optional[int] = None
     ff_act: str = "relu2"
+    latent: Optional[LatentAttnSpec] = None
+    delta: Optional[DeltaSpec] = None
+    moe: Optional[MoESpec] = None
 
 
 @dataclass
@@ -124,6 +198,11 @@ class ModelConfig:
     layer_specs: Optional[List[LayerSpec]] = None
     loop: Optional[LoopSpec] = None
     embed_scale: float = 1.0
+    # arch "pagonex": a causal convolution of ``canon_taps`` taps is added to what every sublayer reads,
+    # a hashed (previous, current) token row is added to the embedding, the logits are scaled
+    canon_taps: int = 0
+    bigram: Optional[dict] = None            # {"buckets", "mul_prev", "mul_cur"}
+    logit_scale: float = 1.0
 
     def layer_runs(self) -> List[tuple]:
         """[(layer index, pass number or None)] in execution order; every run has its own cache."""
@@ -290,9 +369,26 @@ def to_hf_config(cfg: ModelConfig) -> dict:
     raise ValueError(f"no HF config mapping for {cfg.arch}")
 
 
+def checkpoint_shapes(path: str) -> dict:
+    """Tensor name -> shape from the headers of a folder's safetensors files (an 8-byte length, then
+    that many bytes of JSON); no tensor data is read."""
+    import struct
+    shapes = {}
+    for fn in sorted(os.listdir(path)):
+        if fn.endswith(".safetensors"):
+            with open(os.path.join(path, fn), "rb") as f:
+                (n,) = struct.unpack("<Q", f.read(8))
+                for k, v in json.loads(f.read(n)).items():
+                    if k != "__metadata__":
+                        shapes[k] = tuple(v["shape"])
+    return shapes
+
+
 def from_hf_dir(path: str) -> ModelConfig:
     with open(os.path.join(path, "config.json")) as f:
-        return from_hf_config(json.load(f))
+        c = json.load(f)
+    needs_shapes = str(c.get("architecture", "")).lower() == "pagonex"
+    return from_hf_config(c, checkpoint_shapes(path) if needs_shapes else None)
 
 
 def _rope_params(c: dict, default_theta: float, default_partial: float = 1.0):
@@ -369,11 +465,96 @@ def to_nudadra_config(cfg: ModelConfig) -> dict:
     return out
 
 
-def from_hf_config(c: dict) -> ModelConfig:
+def from_pagonex_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
+    """The Pagonex layout of ``config.json``: ``layers`` (``type`` = ``latent_attention`` or
+    ``channel_delta``, ``mixer`` sizes, ``mlp`` = mixture of experts or null), ``canon.taps``,
+    ``embedding.bigram``, ``norm.eps``, ``logit_scale``, ``vocab``, ``width``.  ``shapes`` (tensor
+    name -> shape of the checkpoint) supplies the sizes the config leaves to the tensors: the
+    ranks of the delta layers' decay and gate projections."""
+    specs = []
+    for i, l in enumerate(c["layers"]):
+        m, kind = l["mixer"], l["type"]
+        lat = dl = None
+        if kind == "latent_attention":
+            rot, mask = m.get("rot") or {}, m.get("mask") or {}
+            sc = rot.get("scaling") or None
+            lat = LatentAttnSpec(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+                                 q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
+                                 window=int(mask["size"]) if mask.get("size") is not None else None,
+                                 rot_dims=int(rot.get("dims", m["rot_dim"])), rot_base=float(rot.get("base", 10000.0)),
+                                 rot_scaling=dict(sc, rope_type="yarn") if sc else None,
+                                 kv_from=int(m["kv_from"]) if m.get("kv_from") is not None else None)
+        elif kind == "channel_delta":
+            rank = lambda name, default: int(shapes[f"l{i}.mix.{name}"][0]) if shapes else int(m.get(default, 0) or 16)
+            dl = DeltaSpec(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
+                           vdim=int(m["vdim"]), conv=int(m["conv"]), decay_rank=rank("a1", "decay_rank"),
+                           gate_rank=rank("g1", "gate_rank"))
+        else:
+            raise ValueError(f"unsupported layer type {kind!r}")
+        mlp, moe = l.get("mlp") or None, None
+        if mlp:
+            if mlp.get("kind") != "moe":
+                raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}")
+            r, sh = mlp["router"], mlp.get("shared") or None
+            moe = MoESpec(experts=int(r["experts"]), top=int(r["top"]), scale=float(r.get("scale", 1.0)),
+                          ff=int(mlp["expert"]["ff"]), limit=float(mlp["expert"]["limit"]),
+                          shared_ff=int(sh["ff"]) if sh else 0, shared_limit=float(sh["limit"]) if sh else 0.0)
+        specs.append(LayerSpec(kind, latent=lat, delta=dl, moe=moe))
+    for s in specs:
+        if s.latent is not None and s.latent.kv_from is not None:
+            src = specs[s.latent.kv_from].latent
+            if src is None or src.kv_from is not None or src.cache_dim != s.latent.cache_dim:
+                raise ValueError("kv_from must name a latent-attention layer with its own latent of the same sizes")
+    big = (c.get("embedding") or {}).get("bigram") or None
+    heads = next((s.latent.heads for s in specs if s.latent), specs[0].delta.heads if specs[0].delta else 1)
+    return ModelConfig(arch="pagonex", vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), num_layers=len(specs),
+                       num_heads=heads, num_kv_heads=1, intermediate_size=0, head_dim=1, max_position_embeddings=1 << 20,
+                       norm="layer", norm_eps=float(c["norm"]["eps"]), act="glu_clamp", name=c.get("name", "pagonex"),
+                       layer_specs=specs, canon_taps=int((c.get("canon") or {}).get("taps", 0)),
+                       bigram={k: int(big[k]) for k in ("buckets", "mul_prev", "mul_cur")} if big else None,
+                       logit_scale=float(c.get("logit_scale", 1.0)))
+
+
+def to_pagonex_config(cfg: ModelConfig) -> dict:
+    """Inverse of ``from_pagonex_config`` (the ranks travel as tensor shapes)."""
+    layers = []
+    for s in cfg.layer_specs:
+        if s.latent is not None:
+            a = s.latent
+            m = {"heads": a.heads, "dim": a.dim, "rot_dim": a.rot_dim, "vdim": a.vdim, "q_rank": a.q_rank,
+                 "kv_rank": a.kv_rank, "scale": a.scale, "rot": {"dims": a.rot_dims, "base": a.rot_base}}
+            if a.rot_scaling:
+                m["rot"]["scaling"] = {k: v for k, v in a.rot_scaling.items() if k != "rope_type"}
+            if a.window is not None:
+                m["mask"] = {"size": a.window}
+            if a.kv_from is not None:
+                m["kv_from"] = a.kv_from
+        else:
+            d = s.delta
+            m = {"heads": d.heads, "kv_heads": d.kv_heads, "dim": d.dim, "vdim": d.vdim, "conv": d.conv}
+        mlp = None
+        if s.moe is not None:
+            e = s.moe
+            mlp = {"kind": "moe", "router": {"experts": e.experts, "top": e.top, "scale": e.scale},
+                   "expert": {"ff": e.ff, "limit": e.limit}}
+            if e.shared_ff:
+                mlp["shared"] = {"ff": e.shared_ff, "limit": e.shared_limit}
+        layers.append({"type": s.mixer, "mixer": m, "mlp": mlp})
+    out = {"architecture": "Pagonex", "vocab": cfg.vocab_size, "width": cfg.hidden_size, "layers": layers,
+           "norm": {"eps": cfg.norm_eps}, "canon": {"taps": cfg.canon_taps}, "logit_scale": cfg.logit_scale}
+    if cfg.bigram:
+        out["embedding"] = {"bigram": dict(cfg.bigram)}
+    return out
+
+
+def from_hf_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
     """Map a ``config.json`` onto ModelConfig (Hugging Face ``model_type`` layouts, or an
-    ``architecture`` key naming a per-layer layout)."""
+    ``architecture`` key naming a per-layer layout; ``shapes``: the checkpoint's tensor shapes, for
+    layouts that leave some sizes to them)."""
     if str(c.get("architecture", "")).lower() == "nudadra":
         return from_nudadra_config(c)
+    if str(c.get("architecture", "")).lower() == "pagonex":
+        return from_pagonex_config(c, shapes)
     mt = c.get("model_type")
     eos = c.get("eos_token_id")
     if isinstance(eos, list):

@@ -1,6 +1,12 @@
-"""Layer-spec language models (arch "nudadra"): every layer is described by its own entry of
-``ModelConfig.layer_specs``, a span of layers may run several times in a row, and the residual
-stream is fp32.
+"""Layer-spec language models (arch "nudadra", "pagonex"): every layer is described by its own
+entry of ``ModelConfig.layer_specs``, a span of layers may run several times in a row, and the
+residual stream is fp32.
+
+Per layer (post-norm form, ``PostNormLayer``):  x <- x + LN1(mixer(x + conv1(x))) ;
+x <- x + LN2(ff(x + conv2(x))): the sublayers read the stream itself plus a causal depthwise
+convolution of it over time, and the LayerNorm sits on each sublayer's output.  The mixer is latent
+attention or a gated delta rule (models/mixers.py), the feed-forward a mixture of experts
+(models/moe.py).  The embedding adds a hashed (previous token, token) row; the logits are scaled.
 
 Per layer (parallel form):  h = norm(x) ;  x <- x + mixer(h) + ff(h), with one norm whose gain is a
 single number, a ``ParallelMixer`` (models/mixers.py) and a squared-ReLU feed-forward.  The
@@ -25,8 +31,9 @@ import torch.nn as nn
 
 from ..ops import seqmix
 from .configs import LayerSpec, ModelConfig
-from .layers import Linear, ScalarNorm
-from .mixers import ParallelMixer
+from .layers import Linear, RowLayerNorm, ScalarNorm
+from .mixers import ChannelDeltaMixer, LatentAttention, ParallelMixer
+from .moe import MoEFeedForward
 
 
 class HybridLayer(nn.Module):
@@ -49,6 +56,45 @@ class HybridLayer(nn.Module):
         return self.mix(x, u, meta, run, m)
 
 
+class PostNormLayer(nn.Module):
+    """One mixer (latent attention or gated delta rule) and an optional mixture-of-experts
+    feed-forward, each reading x + conv(x) and adding LayerNorm(its output) to the fp32 stream."""
+
+    def __init__(self, cfg: ModelConfig, spec: LayerSpec, idx: int, dtype, device):
+        super().__init__()
+        W, eps = cfg.hidden_size, cfg.norm_eps
+        self.idx, self.spec, self.dtype = idx, spec, dtype
+        if spec.mixer == "latent_attention":
+            self.mix = LatentAttention(spec.latent, W, eps, dtype, device)
+        elif spec.mixer == "channel_delta":
+            self.mix = ChannelDeltaMixer(spec.delta, W, eps, dtype, device)
+        else:
+            raise ValueError(spec.mixer)
+        taps = cfg.canon_taps
+        P = lambda: nn.Parameter(torch.zeros(W, taps, dtype=torch.float32, device=device), requires_grad=False)
+        self.canon1 = P() if taps else None
+        self.norm1 = RowLayerNorm(W, eps, device)
+        self.ff = MoEFeedForward(spec.moe, W, dtype, device) if spec.moe is not None else None
+        if self.ff is not None:
+            self.canon2 = P() if taps else None
+            self.norm2 = RowLayerNorm(W, eps, device)
+
+    def forward(self, x: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        h = seqmix.canon_conv(x, self.canon1, run.canon1, meta, self.dtype) if self.canon1 is not None else x.to(self.dtype)
+        self.norm1.add_to(x, self.mix(h, meta, run))
+        if self.ff is not None:
+            h = seqmix.canon_conv(x, self.canon2, run.canon2, meta, self.dtype) if self.canon2 is not None \
+                else x.to(self.dtype)
+            shared, parts, wts = self.ff(h)
+            self.norm2.add_to(x, shared, parts, wts)
+        return x
+
+
+def _make_layer(cfg: ModelConfig, spec: LayerSpec, idx: int, dtype, device) -> nn.Module:
+    return HybridLayer(cfg, spec, idx, dtype, device) if spec.mixer == "parallel" else \
+        PostNormLayer(cfg, spec, idx, dtype, device)
+
+
 class HybridLM(nn.Module):
     ragged = True          # runs RaggedMeta steps over a paged cache (engine.ragged)
 
@@ -60,13 +106,17 @@ class HybridLM(nn.Module):
         self.first, self.last = 0, cfg.num_layers
         self.has_embed = self.has_head = True
         self.embed = nn.Parameter(torch.empty(cfg.vocab_size, W, dtype=dtype, device=device), requires_grad=False)
-        self.layers = nn.ModuleList([HybridLayer(cfg, s, i, dtype, device) for i, s in enumerate(cfg.layer_specs)])
+        self.layers = nn.ModuleList([_make_layer(cfg, s, i, dtype, device) for i, s in enumerate(cfg.layer_specs)])
         self.runs = cfg.layer_runs()
+        if cfg.bigram:
+            self.bigram = nn.Parameter(torch.empty(cfg.bigram["buckets"] + 1, W, dtype=dtype, device=device),
+                                       requires_grad=False)
         if cfg.loop is not None:
             self.loop_in = Linear(2 * W, W, False, dtype, device)
             self.loop_step = nn.Parameter(torch.zeros(cfg.loop.times, W, dtype=torch.float32, device=device),
                                           requires_grad=False)
-        self.final_norm = ScalarNorm(cfg.norm_eps, device)
+        self.final_norm = ScalarNorm(cfg.norm_eps, device) if cfg.norm == "rms_scalar" else \
+            RowLayerNorm(W, cfg.norm_eps, device)
         self.lm_head = Linear(W, cfg.vocab_size, False, dtype, device)
 
     @property
@@ -92,7 +142,12 @@ class HybridLM(nn.Module):
         """ids [T] (flat step) -> fp32 logits of ``rows`` (flat row indices; None: every row).
         ``taps`` (a list) receives the residual stream after every run."""
         cfg = self.cfg
-        x0 = seqmix.embedding_scaled(ids, self.embed, cfg.embed_scale)
+        if cfg.bigram:
+            b = cfg.bigram
+            x0 = seqmix.embedding_bigram(ids, meta, self.embed, self.bigram, cache.prev_tok, b["buckets"], b["mul_prev"],
+                                         b["mul_cur"])
+        else:
+            x0 = seqmix.embedding_scaled(ids, self.embed, cfg.embed_scale)
         x = x0.clone() if cfg.loop is not None else x0
         for r, (i, t) in enumerate(self.runs):
             if t is not None and i == cfg.loop.start:
@@ -105,7 +160,8 @@ class HybridLM(nn.Module):
                 return torch.empty(0, cfg.vocab_size, dtype=torch.float32, device=x.device)
             x = x.index_select(0, rows)
         h = self.final_norm(x, self.dtype)
-        return self.lm_head(h).float()
+        logits = self.lm_head(h).float()
+        return logits if cfg.logit_scale == 1.0 else logits.mul_(cfg.logit_scale)
 
 
 # --------------------------------------------------------------------------- weights
@@ -167,6 +223,97 @@ def export_nudadra_tensors(model: HybridLM) -> Dict[str, torch.Tensor]:
     return {k: v.to(dt).contiguous() for k, v in out.items()}
 
 
+def convert_pagonex_tensors(cfg: ModelConfig, t: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    """Checkpoint names of the Pagonex layout (``l<i>.mix.dq``, ``l<i>.mlp.e<k>.gate`` ...) -> this
+    package's parameter names: fused input projections, per-head key / value expansions, stacked
+    expert weights."""
+    out = {"embed": t["embed"], "final_norm.weight": t["final.norm"], "final_norm.bias": t["final.norm.b"],
+           "lm_head.weight": t["head"]}
+    if cfg.bigram:
+        out["bigram"] = t["bigram"]
+    for i, spec in enumerate(cfg.layer_specs):
+        p, o = f"l{i}.", f"layers.{i}."
+        M, m = p + "mix.", o + "mix."
+        for n in ("1", "2") if spec.moe is not None else ("1",):
+            out[o + f"norm{n}.weight"], out[o + f"norm{n}.bias"] = t[p + f"norm{n}"], t[p + f"norm{n}.b"]
+            if cfg.canon_taps:
+                out[o + f"canon{n}"] = t[p + f"canon{n}"]
+        if spec.latent is not None:
+            a = spec.latent
+            out[m + "proj_in.weight"] = torch.cat([t[M + "dq"]] + ([t[M + "dkv"]] if a.kv_from is None else []), 0)
+            out[m + "q_norm"] = t[M + "dq.norm"]
+            if a.kv_from is None:
+                out[m + "kv_norm"] = t[M + "dkv.norm"]
+            out[m + "uq.weight"] = t[M + "uq"]
+            out[m + "uk"] = t[M + "uk"].reshape(a.heads, a.dim, a.kv_rank)
+            out[m + "uv"] = t[M + "uv"].reshape(a.heads, a.vdim, a.kv_rank).transpose(1, 2).contiguous()
+            out[m + "o.weight"] = t[M + "o"]
+        else:
+            d = spec.delta
+            out[m + "proj_in.weight"] = torch.cat([t[M + n] for n in ("q", "k", "v", "b", "a1", "g1")], 0)
+            out[m + "conv_w"] = torch.cat([t[M + n + ".conv"] for n in ("q", "k", "v")], 0)
+            out[m + "a2.weight"], out[m + "g2.weight"] = t[M + "a2"], t[M + "g2"]
+            out[m + "dt_bias"], out[m + "A_log"], out[m + "norm_w"] = t[M + "dt_bias"], t[M + "A_log"], t[M + "norm"]
+            out[m + "o.weight"] = t[M + "o"]
+        if spec.moe is not None:
+            e, F_, f = spec.moe, p + "mlp.", o + "ff."
+            out[f + "router"] = t[F_ + "router"]
+            out[f + "w_gu"] = torch.stack([torch.cat([t[f"{F_}e{k}.gate"], t[f"{F_}e{k}.up"]], 0) for k in range(e.experts)])
+            out[f + "w_down"] = torch.stack([t[f"{F_}e{k}.down"] for k in range(e.experts)])
+            if e.shared_ff:
+                out[f + "shared_gu.weight"] = torch.cat([t[F_ + "shared.gate"], t[F_ + "shared.up"]], 0)
+                out[f + "shared_down.weight"] = t[F_ + "shared.down"]
+    return out
+
+
+def export_pagonex_tensors(model: "HybridLM") -> Dict[str, torch.Tensor]:
+    """Inverse of ``convert_pagonex_tensors`` (checkpoint names, 16-bit storage)."""
+    cfg = model.cfg
+    p = {k: v.detach() for k, v in model.named_parameters()}
+    out = {"embed": p["embed"], "final.norm": p["final_norm.weight"], "final.norm.b": p["final_norm.bias"],
+           "head": p["lm_head.weight"]}
+    if cfg.bigram:
+        out["bigram"] = p["bigram"]
+    for i, spec in enumerate(cfg.layer_specs):
+        q, o = f"l{i}.", f"layers.{i}."
+        M, m = q + "mix.", o + "mix."
+        for n in ("1", "2") if spec.moe is not None else ("1",):
+            out[q + f"norm{n}"], out[q + f"norm{n}.b"] = p[o + f"norm{n}.weight"], p[o + f"norm{n}.bias"]
+            if cfg.canon_taps:
+                out[q + f"canon{n}"] = p[o + f"canon{n}"]
+        if spec.latent is not None:
+            a = spec.latent
+            w = p[m + "proj_in.weight"]
+            out[M + "dq"], out[M + "dq.norm"] = w[:a.q_rank], p[m + "q_norm"]
+            if a.kv_from is None:
+                out[M + "dkv"], out[M + "dkv.norm"] = w[a.q_rank:], p[m + "kv_norm"]
+            out[M + "uq"] = p[m + "uq.weight"]
+            out[M + "uk"] = p[m + "uk"].reshape(a.heads * a.dim, a.kv_rank)
+            out[M + "uv"] = p[m + "uv"].transpose(1, 2).reshape(a.heads * a.vdim, a.kv_rank)
+            out[M + "o"] = p[m + "o.weight"]
+        else:
+            d = spec.delta
+            for n, part in zip(("q", "k", "v", "b", "a1", "g1"), torch.split(p[m + "proj_in.weight"], list(d.in_sizes), 0)):
+                out[M + n] = part
+            GN = d.kv_heads * d.dim
+            for n, part in zip(("q", "k", "v"), torch.split(p[m + "conv_w"], [GN, GN, d.heads * d.vdim], 0)):
+                out[M + n + ".conv"] = part
+            out[M + "a2"], out[M + "g2"] = p[m + "a2.weight"], p[m + "g2.weight"]
+            out[M + "dt_bias"], out[M + "A_log"], out[M + "norm"] = p[m + "dt_bias"], p[m + "A_log"], p[m + "norm_w"]
+            out[M + "o"] = p[m + "o.weight"]
+        if spec.moe is not None:
+            e, F_, f = spec.moe, q + "mlp.", o + "ff."
+            out[F_ + "router"] = p[f + "router"]
+            for k in range(e.experts):
+                out[f"{F_}e{k}.gate"], out[f"{F_}e{k}.up"] = p[f + "w_gu"][k, :e.ff], p[f + "w_gu"][k, e.ff:]
+                out[f"{F_}e{k}.down"] = p[f + "w_down"][k]
+            if e.shared_ff:
+                out[F_ + "shared.gate"], out[F_ + "shared.up"] = p[f + "shared_gu.weight"][:e.shared_ff], \
+                    p[f + "shared_gu.weight"][e.shared_ff:]
+                out[F_ + "shared.down"] = p[f + "shared_down.weight"]
+    return {k: v.to(torch.bfloat16).contiguous() for k, v in out.items()}
+
+
 @torch.no_grad()
 def load_into_hybrid(model: HybridLM, tensors: Dict[str, torch.Tensor]) -> HybridLM:
     missing = []
@@ -204,6 +351,16 @@ def init_random_hybrid_(model: HybridLM, seed: int = 0) -> HybridLM:
             v = 1.0 + 0.1 * r(*p.shape)
         elif leaf == "conv_w":
             v = r(*p.shape) / p.shape[1] ** 0.5
+        elif leaf in ("uk", "uv", "w_gu", "w_down"):     # stacked [.., out, in] or [heads, in, out] expansions
+            v = r(*p.shape) / p.shape[-1 if leaf in ("w_gu", "w_down") else 1] ** 0.5
+        elif leaf == "router" or name == "bigram":
+            v = r(*p.shape) * (0.5 if name == "bigram" else 1.0)
+        elif leaf in ("q_norm", "kv_norm"):
+            v = 1.0 + 0.1 * r(*p.shape)
+        elif leaf in ("canon1", "canon2"):
+            v = 0.3 * r(*p.shape)
+        elif leaf == "bias" and p.dim() == 1:            # LayerNorm biases
+            v = 0.1 * r(*p.shape)
         else:                                            # conv_b, loop_step
             v = 0.1 * r(*p.shape)
         p.copy_(v.to(torch.bfloat16).to(p.dtype))

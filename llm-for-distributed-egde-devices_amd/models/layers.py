@@ -269,6 +269,24 @@ class ScalarNorm(nn.Module):
         return ops.seqmix.scalar_rms_norm(x, self.weight, self.eps, out_dtype)
 
 
+class RowLayerNorm(nn.Module):
+    """LayerNorm with weight and bias over fp32 rows (the residual stream of the layer-spec models),
+    rows of the consumer's dtype out; ``add_to`` instead adds the normed rows into an fp32 stream in
+    place (a norm on a sublayer's output), optionally over y + sum_k part_w[:, k] parts[:, k]."""
+
+    def __init__(self, width: int, eps: float, device=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32, device=device), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(width, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, x: torch.Tensor, out_dtype=torch.bfloat16) -> torch.Tensor:
+        return ops.seqmix.layer_norm_rows(x, self.weight, self.bias, self.eps, out_dtype)
+
+    def add_to(self, x: torch.Tensor, y, parts=None, part_w=None) -> torch.Tensor:
+        return ops.seqmix.layer_norm_residual(x, y, self.weight, self.bias, self.eps, parts, part_w)
+
+
 def act_fn(x, act: str, quant: bool):
     if quant:
         q, s = ops.activation_quant(x, act)

@@ -119,3 +119,102 @@ class ParallelMixer(nn.Module):
         a = self.left(u, 0, meta, run)
         r = self.right(u, sum(self.left.spec.proj_sizes), meta, run)
         return seqmix.combine_residual(x, a, r, self.left_out, self.right_out, self.eps, extra)
+
+
+def _shared_rope(store, key_spec, n: int, device) -> Optional[torch.Tensor]:
+    """cos / sin rows for positions [0, n) from the table shared by every mixer with the same rotation
+    constants (``key_spec``: rot_dims, base, scaling), grown by doubling."""
+    dims, base, scaling = key_spec
+    if not dims:
+        return None
+    tab = store.get("tab")
+    if tab is None or tab.shape[0] < n or tab.device != torch.device(device):
+        key = (dims, base, tuple(sorted((scaling or {}).items())), str(torch.device(device)))
+        tab = _ROPE_TABLES.get(key)
+        if tab is None or tab.shape[0] < n:
+            from .. import ops
+            rows = 2048
+            while rows < n:
+                rows *= 2
+            if tab is not None:
+                _ROPE_RETIRED.append(tab)
+            tab = _ROPE_TABLES[key] = ops.rope_tables(dims, rows, base, scaling, device=device)
+        store["tab"] = tab
+    return tab
+
+
+class LatentAttention(nn.Module):
+    """Softmax attention whose keys and values are expanded per head from one cached latent.
+
+    Cached per token: c = rms(W_dkv h)[: kv_rank] w and one rotated key part of R numbers shared by
+    the heads.  Head h scores q_h . (W_uk,h c) + q_rot,h . k_rot; since q_h . (W_uk,h c) =
+    (W_uk,h^T q_h) . c, the queries are carried through the key expansion once per token and the
+    attention runs as one kv head of size kv_rank + R over the cached rows themselves, with the
+    latent as the value; each head's weighted latent is then expanded by W_uv,h.  The cache is read
+    once for all heads and nothing per head is stored.  A layer with ``kv_from`` reads another
+    layer's cached rows and has no down projection of its own."""
+
+    def __init__(self, spec, width: int, eps: float, dtype, device):
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        s = spec
+        P = lambda *shape: nn.Parameter(torch.zeros(*shape, dtype=torch.float32, device=device), requires_grad=False)
+        self.own_kv = s.kv_from is None
+        # rows: query latent | (key / value latent | shared key part)
+        self.proj_in = Linear(width, s.q_rank + (s.cache_dim if self.own_kv else 0), False, dtype, device)
+        self.q_norm = P(s.q_rank)
+        self.kv_norm = P(s.kv_rank) if self.own_kv else None
+        self.uq = Linear(s.q_rank, s.heads * (s.dim + s.rot_dim), False, dtype, device)
+        self.uk = nn.Parameter(torch.zeros(s.heads, s.dim, s.kv_rank, dtype=dtype, device=device), requires_grad=False)
+        self.uv = nn.Parameter(torch.zeros(s.heads, s.kv_rank, s.vdim, dtype=dtype, device=device), requires_grad=False)
+        self.o = Linear(s.heads * s.vdim, width, False, dtype, device)
+        self._rope = {}
+
+    def forward(self, h: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        s = self.spec
+        T, H = h.shape[0], s.heads
+        u = self.proj_in(h)
+        cq = seqmix.rms_norm_cols(u, 0, s.q_rank, self.q_norm, self.eps, h.dtype)
+        q = self.uq(cq).view(T, H, s.dim + s.rot_dim)
+        q_lat = torch.bmm(q[:, :, :s.dim].transpose(0, 1), self.uk).transpose(0, 1)      # [T, H, kv_rank]
+        rope = _shared_rope(self._rope, (s.rot_dims, s.rot_base, s.rot_scaling), meta.max_keys, h.device)
+        qc = seqmix.latent_write(u if self.own_kv else None, s.q_rank, self.kv_norm, self.eps, q, q_lat, meta, rope,
+                                 run.lat, s.kv_rank, s.rot_dims)
+        a = seqmix.window_pool_attention(qc, None, run.lat, run.lat[..., :s.kv_rank], None, None, meta, s.scale,
+                                         s.window, None)                                # [T, H * kv_rank]
+        v = torch.bmm(a.view(T, H, s.kv_rank).transpose(0, 1), self.uv).transpose(0, 1)  # [T, H, vdim]
+        return self.o(v.reshape(T, H * s.vdim))
+
+
+class ChannelDeltaMixer(nn.Module):
+    """Gated delta rule with a decay per head and key channel: convolution + silu over q | k | v,
+    unit-length q and k, beta = sigmoid(W_b h), decays exp(-exp(A_log) softplus(W_a2 W_a1 h + bias)),
+    the recurrence over a [dim, vdim] fp32 state per head, a per-head RMS norm with a sigmoid output
+    gate W_g2 W_g1 h, and the output projection.  One fused GEMM produces q | k | v | beta and the two
+    low-rank projections' inner rows."""
+
+    def __init__(self, spec, width: int, eps: float, dtype, device):
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        s = spec
+        P = lambda *shape: nn.Parameter(torch.zeros(*shape, dtype=torch.float32, device=device), requires_grad=False)
+        self.proj_in = Linear(width, sum(s.in_sizes), False, dtype, device)
+        self.conv_w = P(s.conv_channels, s.conv)
+        self.register_buffer("conv_b", torch.zeros(s.conv_channels, dtype=torch.float32, device=device),
+                             persistent=False)             # this mixer's convolutions have no bias
+        self.a2 = Linear(s.decay_rank, s.heads * s.dim, False, dtype, device)
+        self.g2 = Linear(s.gate_rank, s.heads * s.vdim, False, dtype, device)
+        self.dt_bias, self.A_log, self.norm_w = P(s.heads * s.dim), P(s.heads), P(s.vdim)
+        self.o = Linear(s.heads * s.vdim, width, False, dtype, device)
+
+    def forward(self, h: torch.Tensor, meta: seqmix.RaggedMeta, run) -> torch.Tensor:
+        s = self.spec
+        nq, nk, nv, nb, na, ng = s.in_sizes
+        u = self.proj_in(h)
+        C = s.conv_channels
+        qkv = seqmix.conv_silu(u, 0, C, self.conv_w, self.conv_b, run.conv, meta)
+        a = seqmix.linear_f32(u[:, C + nb:C + nb + na], self.a2.weight)                 # fp32: it feeds the decays
+        z = self.g2(u[:, C + nb + na:C + nb + na + ng])
+        prep = seqmix.delta_prepare(qkv, u, C, a, self.dt_bias, self.A_log, s.heads, s.kv_heads, s.dim)
+        y = seqmix.delta_rule_scan(prep, qkv, run.ssm, meta, s.heads, s.kv_heads, s.dim, s.vdim)
+        return self.o(seqmix.head_norm_gate(y, z, self.norm_w, s.heads, self.eps, h.dtype))

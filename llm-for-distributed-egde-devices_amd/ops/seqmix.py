@@ -350,3 +350,244 @@ def ssd_scan(xbc: torch.Tensor, u: torch.Tensor, dt0: int, dt_bias, A_log, D, st
             y[off + t] = (torch.einsum("hnp,hn->hp", S, C[t]) + D.float()[:, None] * x[t]).reshape(inner)
         state[slot] = S
     return y
+
+
+# --------------------------------------------------------------------------- post-norm layers: rows
+def embedding_bigram(ids: torch.Tensor, meta: RaggedMeta, table: torch.Tensor, bigram: torch.Tensor,
+                     prev_tok: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int) -> torch.Tensor:
+    """fp32 rows ``table[id] + bigram[(prev * mul_prev + id * mul_cur) mod buckets]``; a sequence's
+    first token takes row ``buckets``.  ``prev_tok`` int64 [slots] holds each slot's last token
+    (read by a portion that continues a sequence, left at the portion's last token)."""
+    if _gpu(table):
+        return _ext().sm_embed_bigram(ids.long().contiguous(), table, bigram, prev_tok, meta.tok_seq, meta.tok_pos,
+                                      meta.seq_slot, meta.seq_start, meta.seq_len, meta.seq_off, int(meta.n),
+                                      int(buckets), int(mul_prev), int(mul_cur))
+    ids = ids.long()
+    out = table[ids].float()
+    for slot, start, n, off in meta.host:
+        cur = ids[off:off + n]
+        prev = torch.cat([prev_tok[slot:slot + 1] if start > 0 else cur[:1], cur[:-1]])
+        row = (prev * mul_prev + cur * mul_cur) % buckets
+        if start == 0:
+            row[0] = buckets
+        out[off:off + n] += bigram[row].float()
+        prev_tok[slot] = cur[-1]
+    return out
+
+
+def canon_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, meta: RaggedMeta, out_dtype) -> torch.Tensor:
+    """x + causal depthwise convolution of x over time, fp32 [T, W] in, ``out_dtype`` out.  weight fp32
+    [W, taps] (last tap = the current token), state fp32 [slots, taps - 1, W] = each slot's last inputs
+    (taken as zero by a portion starting at position 0; left at the portion's last taps - 1 inputs)."""
+    taps = weight.shape[1]
+    if _gpu(x):
+        return _ext().sm_canon(x, weight, state, meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.seq_start, meta.seq_len,
+                               meta.seq_off, int(meta.n), out_dtype == torch.float32)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    W = x.shape[1]
+    for slot, start, n, off in meta.host:
+        xs = x[off:off + n]
+        hist = state[slot, :taps - 1] if start > 0 else torch.zeros(taps - 1, W, device=x.device)
+        xin = torch.cat([hist, xs], 0)
+        win = xin.unfold(0, taps, 1)                              # [n, W, taps]
+        out[off:off + n] = (xs + (win * weight[None]).sum(-1)).to(out_dtype)
+        if taps > 1:
+            state[slot, :taps - 1] = xin[xin.shape[0] - (taps - 1):]
+    return out
+
+
+def layer_norm_rows(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """LayerNorm (mean and variance over the width, fp32) of fp32 rows, stored as ``out_dtype``."""
+    if _gpu(x):
+        return _ext().sm_layer_norm(x, weight, bias, float(eps), out_dtype == torch.float32)
+    return F.layer_norm(x, (x.shape[-1],), weight.float(), bias.float(), eps).to(out_dtype)
+
+
+def layer_norm_residual(x: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor, eps: float,
+                        parts: Optional[torch.Tensor] = None, part_w: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x (fp32 [T, W], in place) += LayerNorm(y) weight + bias, statistics in fp32.  ``parts``
+    [T, K, W] with ``part_w`` fp32 [T, K]: the normed row is y + sum_k part_w[:, k] parts[:, k] (a
+    mixture's weighted expert outputs beside its shared expert, summed in fp32 in k order; y None:
+    the parts alone)."""
+    if _gpu(x):
+        _ext().sm_ln_residual(x, y, weight, bias, float(eps), parts, part_w)
+        return x
+    v = y.float() if y is not None else torch.zeros_like(x)
+    if parts is not None:
+        for k in range(parts.shape[1]):
+            v = v + part_w[:, k:k + 1] * parts[:, k].float()
+    x.add_(F.layer_norm(v, (v.shape[-1],), weight.float(), bias.float(), eps))
+    return x
+
+
+def rms_norm_cols(u: torch.Tensor, c0: int, C: int, weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    """RMS norm (fp32) of columns [c0, c0 + C) of u [T, *] times weight [C], contiguous ``out_dtype``."""
+    if _gpu(u):
+        return _ext().sm_rms_cols(u, int(c0), int(C), weight, float(eps), out_dtype == torch.float32)
+    v = u[:, c0:c0 + C].float()
+    return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
+
+
+def glu_clamp(u: torch.Tensor, ff: int, limit: float) -> torch.Tensor:
+    """u [T, gate | up] -> g sigmoid(1.702 g) (up + 1) with g = min(gate, limit), up clamped to
+    +-limit (fp32 math, stored in u's dtype)."""
+    if _gpu(u):
+        return _ext().sm_glu_clamp(u, int(ff), float(limit))
+    g = u[:, :ff].float().clamp(max=limit)
+    up = u[:, ff:2 * ff].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (up + 1)).to(u.dtype)
+
+
+# --------------------------------------------------------------------------- latent attention
+def _rotate_pairs(x, cs, dims):
+    """x [.., n] with neighbouring coordinates (2i, 2i + 1) of the first ``dims`` turned by cs [.., dims/2, 2]."""
+    u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+    c, s = cs[..., 0], cs[..., 1]
+    rot = torch.stack([u * c - v * s, v * c + u * s], -1).flatten(-2)
+    return torch.cat([rot, x[..., dims:]], -1)
+
+
+def latent_write(u: Optional[torch.Tensor], c0: int, weight: Optional[torch.Tensor], eps: float, q: torch.Tensor,
+                 q_lat: torch.Tensor, meta: RaggedMeta, rope: Optional[torch.Tensor], pages: torch.Tensor, kv_rank: int,
+                 rot_dims: int) -> torch.Tensor:
+    """The cached side and the query side of latent attention, before the scores.
+
+    ``u`` columns [c0, c0 + kv_rank + R) hold a token's down-projected latent | shared key part: the
+    latent is RMS-normed (fp32) times ``weight``, the key part is rotated at the token's position,
+    and both go to the token's row of ``pages`` [pages, page, 1, kv_rank + R].  ``u`` None: the pages
+    already hold them (a layer that reads another layer's cache).  Returns the queries against that
+    row layout, [T, H, kv_rank + R]: ``q_lat`` [T, H, kv_rank] (the unrotated query parts carried
+    through the key expansion) beside the rotated last R coordinates of ``q`` [T, H, D + R]."""
+    T, H, DR = q.shape
+    R = pages.shape[-1] - kv_rank
+    if _gpu(q):
+        return _ext().sm_latent_write(u, int(c0), weight, float(eps), q, q_lat, meta.tok_seq, meta.tok_pos, meta.seq_slot,
+                                      meta.page_table, rope if rot_dims else None, pages, int(kv_rank), int(rot_dims))
+    pos = meta.tok_pos.long()
+    cs = rope[pos] if (rope is not None and rot_dims) else None
+    if u is not None:
+        d = u[:, c0:c0 + kv_rank + R].float()
+        c = d[:, :kv_rank]
+        c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+        kr = d[:, kv_rank:]
+        if cs is not None:
+            kr = _rotate_pairs(kr, cs, rot_dims)
+        slot = meta.seq_slot.long()[meta.tok_seq.long()]
+        pid = meta.page_table[slot, pos // meta.page].long()
+        pages[pid, pos % meta.page, 0] = torch.cat([c, kr], -1).to(pages.dtype)
+    qr = q[:, :, DR - R:].float()
+    if cs is not None:
+        qr = _rotate_pairs(qr, cs[:, None], rot_dims)
+    return torch.cat([q_lat.float(), qr], -1).to(q.dtype)
+
+
+# --------------------------------------------------------------------------- gated delta rule
+def delta_prepare(qkv: torch.Tensor, u: torch.Tensor, b0: int, a: torch.Tensor, dt_bias: torch.Tensor,
+                  A_log: torch.Tensor, heads: int, kv_heads: int, N: int):
+    """What the delta-rule recurrence reads, all fp32: unit-length q (times N^-1/2) and k
+    [T, kv heads, N] from the first 2 kv_heads N columns of ``qkv`` (after convolution + silu), the
+    decays exp(-exp(A_log) softplus(a + dt_bias)) [T, heads, N], and beta = sigmoid of columns
+    [b0, b0 + heads) of u.  Returns one tensor [T, 2 kv_heads N + heads N + heads]: q | k | decay | beta."""
+    if _gpu(qkv):
+        return _ext().sm_delta_prep(qkv, u, int(b0), a, dt_bias, A_log, int(heads), int(kv_heads), int(N))
+    T, GN = qkv.shape[0], kv_heads * N
+    unit = lambda x: x * torch.rsqrt(x.pow(2).sum(-1, keepdim=True) + 1e-6)
+    q = unit(qkv[:, :GN].float().view(T, kv_heads, N)) * N ** -0.5
+    k = unit(qkv[:, GN:2 * GN].float().view(T, kv_heads, N))
+    sp = F.softplus(a.float() + dt_bias.float(), threshold=1e9).view(T, heads, N)
+    g = torch.exp(-torch.exp(A_log.float())[None, :, None] * sp)
+    beta = torch.sigmoid(u[:, b0:b0 + heads].float())
+    return torch.cat([q.reshape(T, GN), k.reshape(T, GN), g.reshape(T, heads * N), beta], -1)
+
+
+def delta_rule_scan(prep: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, meta: RaggedMeta, heads: int,
+                    kv_heads: int, N: int, P: int) -> torch.Tensor:
+    """The gated delta rule, token by token in fp32.  ``prep`` from ``delta_prepare``; the values are
+    columns [2 kv_heads N, ..) of ``qkv``.  Per head, with S [N, P]:  S <- g * S (rows) ;
+    w = beta (v - S^T k) ;  S <- S + k w^T ;  o = S^T q.  state [slots, heads, N, P] fp32 is read
+    (zero for a portion starting at 0) and left at the portion's end.  Returns o fp32 [T, heads P]."""
+    if _gpu(prep):
+        return _ext().sm_delta_scan(prep, qkv, state, meta.seq_slot, meta.seq_start, meta.seq_len, meta.seq_off,
+                                    int(meta.n), int(heads), int(kv_heads), int(N), int(P))
+    T, GN, rep = prep.shape[0], kv_heads * N, heads // kv_heads
+    out = torch.empty(T, heads * P, dtype=torch.float32, device=prep.device)
+    for slot, start, n, off in meta.host:
+        pr = prep[off:off + n]
+        q = pr[:, :GN].view(n, kv_heads, N).repeat_interleave(rep, 1)
+        k = pr[:, GN:2 * GN].view(n, kv_heads, N).repeat_interleave(rep, 1)
+        g = pr[:, 2 * GN:2 * GN + heads * N].view(n, heads, N)
+        beta = pr[:, 2 * GN + heads * N:]
+        v = qkv[off:off + n, 2 * GN:2 * GN + heads * P].float().view(n, heads, P)
+        S = state[slot].clone() if start > 0 else torch.zeros_like(state[slot])
+        for t in range(n):
+            S = g[t][:, :, None] * S
+            w = beta[t][:, None] * (v[t] - torch.einsum("hnp,hn->hp", S, k[t]))
+            S = S + k[t][:, :, None] * w[:, None, :]
+            out[off + t] = torch.einsum("hnp,hn->hp", S, q[t]).reshape(heads * P)
+        state[slot] = S
+    return out
+
+
+def head_norm_gate(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, heads: int, eps: float, out_dtype) -> torch.Tensor:
+    """Each head's part of y (fp32 [T, heads P]) divided by its root mean square, times weight [P]
+    (shared by the heads), times sigmoid(z) (z [T, heads P], a possibly strided view)."""
+    if _gpu(y):
+        return _ext().sm_head_norm_gate(y, z, weight, int(heads), float(eps), out_dtype == torch.float32)
+    T, C = y.shape
+    g = y.view(T, heads, C // heads)
+    g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    return (g.view(T, C) * torch.sigmoid(z.float())).to(out_dtype)
+
+
+# --------------------------------------------------------------------------- mixture of experts
+def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float):
+    """Softmax router in fp32 over h [T, W] (router fp32 [E, W]): the ``top`` largest scores of every
+    token, divided by their sum (+ 1e-20) and multiplied by ``scale``.  Returns (expert ids int32
+    [T, top], weights fp32 [T, top]), largest first."""
+    if _gpu(h):
+        return _ext().sm_moe_route(h, router, int(top), float(scale))
+    s = torch.softmax(h.float() @ router.float().t(), -1)
+    w, idx = torch.topk(s, top, -1)
+    return idx.int(), w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+
+
+MOE_GEMM_MIN = int(__import__("os").environ.get("EDGELLM_MOE_GEMM_MIN", "64"))
+
+
+def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gu: torch.Tensor, w_down: torch.Tensor, limit: float) -> torch.Tensor:
+    """Every token's chosen experts: h [T, W], idx int32 [T, top], w_gu [E, 2 ff, W] (gate rows, then
+    up rows), w_down [E, W, ff] -> the experts' outputs [T, top, W] (not yet weighted)."""
+    T, top = idx.shape
+    E, ff2, W = w_gu.shape
+    if _gpu(h):
+        if T >= MOE_GEMM_MIN:
+            return _moe_experts_sorted(h, idx, w_gu, w_down, limit)
+        return _ext().sm_moe_experts(h, idx, w_gu, w_down, float(limit))
+    out = torch.zeros(T, top, w_down.shape[1], dtype=h.dtype, device=h.device)
+    for e in idx.unique().tolist():
+        t, k = (idx == e).nonzero(as_tuple=True)
+        y = glu_clamp(F.linear(h[t], w_gu[e]), ff2 // 2, limit)
+        out[t, k] = F.linear(y, w_down[e])
+    return out
+
+
+def _moe_experts_sorted(h, idx, w_gu, w_down, limit):
+    """Prompt-sized steps: (token, choice) pairs sorted by expert, one pair of vendor GEMMs per expert
+    over its rows (the counts cross to the host once per call)."""
+    T, top = idx.shape
+    E, ff2, W = w_gu.shape
+    flat = idx.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=E).tolist()
+    rows = h.index_select(0, order // top)
+    y = torch.empty(T * top, ff2 // 2, dtype=h.dtype, device=h.device)
+    o = torch.empty(T * top, w_down.shape[1], dtype=h.dtype, device=h.device)
+    a = 0
+    for e, n in enumerate(counts):
+        if n:
+            y[a:a + n] = glu_clamp(F.linear(rows[a:a + n], w_gu[e]), ff2 // 2, limit)
+            torch.mm(y[a:a + n], w_down[e].t(), out=o[a:a + n])
+            a += n
+    out = torch.empty_like(o)
+    out[order] = o
+    return out.view(T, top, -1)
