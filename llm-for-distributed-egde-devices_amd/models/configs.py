@@ -481,7 +481,8 @@ def from_pagonex_config(c: dict, shapes: Optional[dict] = None) -> ModelConfig:
             lat = LatentAttnSpec(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
                                  q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]), scale=float(m["scale"]),
                                  window=int(mask["size"]) if mask.get("size") is not None else None,
-                                 rot_dims=int(rot.get("dims", m["rot_dim"])), rot_base=float(rot.get("base", 10000.0)),
+                                 rot_dims=int(rot.get("dims", m["rot_dim"])) if rot else 0,
+                                 rot_base=float(rot.get("base", 10000.0)),
                                  rot_scaling=dict(sc, rope_type="yarn") if sc else None,
                                  kv_from=int(m["kv_from"]) if m.get("kv_from") is not None else None)
         elif kind == "channel_delta":
@@ -522,8 +523,10 @@ def to_pagonex_config(cfg: ModelConfig) -> dict:
         if s.latent is not None:
             a = s.latent
             m = {"heads": a.heads, "dim": a.dim, "rot_dim": a.rot_dim, "vdim": a.vdim, "q_rank": a.q_rank,
-                 "kv_rank": a.kv_rank, "scale": a.scale, "rot": {"dims": a.rot_dims, "base": a.rot_base}}
-            if a.rot_scaling:
+                 "kv_rank": a.kv_rank, "scale": a.scale}
+            if a.rot_dims:
+                m["rot"] = {"dims": a.rot_dims, "base": a.rot_base}
+            if a.rot_dims and a.rot_scaling:
                 m["rot"]["scaling"] = {k: v for k, v in a.rot_scaling.items() if k != "rope_type"}
             if a.window is not None:
                 m["mask"] = {"size": a.window}

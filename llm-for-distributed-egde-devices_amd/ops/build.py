@@ -78,7 +78,7 @@ def _build_target(target: str, verbose: bool, jobs: int) -> str:
     os.makedirs(build_dir, exist_ok=True)
     inc, lib, abi = _torch_paths()
     py_inc = sysconfig.get_paths()["include"]
-    header_deps = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    header_deps = [os.path.join(d, f) for d in {CSRC, src_dir} for f in os.listdir(d) if f.endswith(".h")]
     jobs_list = []
     objs = []
     for f in sorted(os.listdir(src_dir)):

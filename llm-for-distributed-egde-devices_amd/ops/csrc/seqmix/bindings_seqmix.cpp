@@ -27,13 +27,13 @@ int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, co
 int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
-                      int window, int pool, int f32, int nsplit, float* part, hipStream_t st);
-size_t edge_sm_attention_part_floats(int rows, int H, int G, int Dv, int nsplit);
+                      int window, int pool, int f32, int nsplit, float* part, int kld, int vld, hipStream_t st);
+size_t edge_sm_attention_part_floats(int rows, int H, int G, int D, int Dv, int nsplit);
 int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp,
                            const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
                            const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
                            int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
-                           int pool, hipStream_t st);
+                           int pool, int kld, int vld, hipStream_t st);
 int edge_sm_conv_silu(const void* u, int ld, int c0, int C, const float* w, const float* bias, void* state,
                       const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_start,
                       const int* seq_len, const int* seq_off, void* out, int rows, int n, int taps, int f32,
@@ -45,6 +45,35 @@ int edge_sm_ssd_chunked(const void* xbc, int Cx, const void* u, int ld, int dt0,
                         const float* A_log, const float* Dp, float* state, const int* seq_slot, const int* seq_start,
                         const int* seq_len, const int* seq_off, float* y, float* sloc, float* cdec, int n,
                         int max_chunks, int Hs, int P, int N, int groups, int f32, hipStream_t st);
+int edge_sm_embed_bigram(const int64_t* ids, const void* table, const void* bigram, int64_t* prev_tok, const int* tok_seq,
+                         const int* tok_pos, const int* seq_slot, const int* seq_start, const int* seq_len,
+                         const int* seq_off, float* out, int rows, int n, int W, int V, long buckets, long mul_prev,
+                         long mul_cur, int f32, hipStream_t st);
+int edge_sm_canon(const float* x, int W, const float* w, float* state, const int* tok_seq, const int* tok_pos,
+                  const int* seq_slot, const int* seq_start, const int* seq_len, const int* seq_off, void* out, int rows,
+                  int n, int taps, int max_len, int f32, hipStream_t st);
+int edge_sm_layer_norm(const float* x, const float* w, const float* b, void* y, int rows, int W, float eps, int f32,
+                       hipStream_t st);
+int edge_sm_ln_residual(float* x, const void* y, const void* parts, const float* pw, int K, const float* w, const float* b,
+                        int rows, int W, float eps, int f32, hipStream_t st);
+int edge_sm_rms_cols(const void* u, int ld, int c0, int C, const float* w, void* y, int rows, float eps, int f32,
+                     hipStream_t st);
+int edge_sm_head_norm_gate(const float* y, const void* z, int z_ld, const float* w, void* out, int rows, int H, int P,
+                           float eps, int f32, hipStream_t st);
+int edge_sm_glu_clamp(const void* u, int ld, void* y, int rows, int ff, float limit, int f32, hipStream_t st);
+int edge_sm_latent_write(const void* u, int ld, int c0, const float* w, float eps, const void* q, const void* q_lat,
+                         long ql_t, long ql_h, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
+                         int ptab_ld, const float* cs, void* pages, void* qc, int rows, int H, int D, int R, int kvr, int rot,
+                         int page, int f32, hipStream_t st);
+int edge_sm_delta_prep(const void* qkv, int Cq, const void* u, int ld, int b0, const float* a, const float* dt_bias,
+                       const float* A_log, float* prep, int rows, int H, int G, int N, int f32, hipStream_t st);
+int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, float* state, const int* seq_slot,
+                       const int* seq_start, const int* seq_len, const int* seq_off, float* y, int n, int H, int G, int N,
+                       int P, int f32, hipStream_t st);
+int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, int* idx, float* wts, int rows,
+                      int f32, hipStream_t st);
+int edge_sm_moe_experts(const void* h, int W, const int* idx, int top, const void* w_gu, const void* w_down, int ff,
+                        float limit, void* y, void* out, int rows, int f32, hipStream_t st);
 }
 
 namespace {
@@ -211,9 +240,15 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
   chk_i32(seq_slot, "seq_slot");
   chk_table(ptab);
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && is_act(q), "q: [T, H, D]");
-  TORCH_CHECK(kp.scalar_type() == q.scalar_type() && vp.scalar_type() == q.scalar_type() && kp.is_contiguous() &&
-                  vp.is_contiguous() && kp.dim() == 4 && vp.dim() == 4 && kp.size(3) == q.size(2), "pages: [pages, page, G, D]");
+  TORCH_CHECK(kp.scalar_type() == q.scalar_type() && vp.scalar_type() == q.scalar_type() && kp.dim() == 4 &&
+                  vp.dim() == 4 && kp.size(3) == q.size(2), "pages: [pages, page, G, D]");
   const int64_t T = q.size(0), H = q.size(1), D = q.size(2), page = kp.size(1), G = kp.size(2), Dv = vp.size(3);
+  // rows of a page lie kld / vld elements apart (a value that is a slice of the key row shares its stride);
+  // pages are dense runs of rows, heads dense inside a row
+  const int64_t kld = kp.stride(1), vld = vp.stride(1);
+  TORCH_CHECK(kp.stride(3) == 1 && vp.stride(3) == 1 && (G == 1 || (kp.stride(2) == D && vp.stride(2) == Dv)) &&
+                  kp.stride(0) == page * kld && vp.stride(0) == page * vld && kld >= G * D && vld >= G * Dv &&
+                  vp.size(0) == kp.size(0) && vp.size(1) == page && vp.size(2) == G, "pages: rows must be dense runs");
   TORCH_CHECK(max_keys <= ptab.size(1) * page, "page table too short for the step");
   int gate_ld = 0, PB = 0;
   if (gate) {
@@ -244,7 +279,7 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
                                           seq_start->data_ptr<int>(), seq_len->data_ptr<int>(), seq_off->data_ptr<int>(),
                                           ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)n, (int)qtiles,
                                           (int)H, (int)G, (int)D, (int)Dv, (int)page, PB, (float)scale, (int)window,
-                                          PB ? (int)pool : 0, stream());
+                                          PB ? (int)pool : 0, (int)kld, (int)vld, stream());
     if (rc != 1) {
       check(rc, "sm_attention_mfma");
       return out;
@@ -259,14 +294,14 @@ at::Tensor sm_attention(const at::Tensor& q, const std::optional<at::Tensor>& ga
   }
   at::Tensor part;
   if (nsplit > 1)
-    part = at::empty({(int64_t)edge_sm_attention_part_floats((int)T, (int)H, (int)G, (int)Dv, nsplit)},
+    part = at::empty({(int64_t)edge_sm_attention_part_floats((int)T, (int)H, (int)G, (int)D, (int)Dv, nsplit)},
                      q.options().dtype(at::kFloat));
   check(edge_sm_attention(q.data_ptr(), gate ? gate->data_ptr() : nullptr, gate_ld, kp.data_ptr(), vp.data_ptr(),
                           PB ? kb->data_ptr<float>() : nullptr, PB ? vb->data_ptr<float>() : nullptr,
                           tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),
                           ptab.data_ptr<int>(), (int)ptab.stride(0), out.data_ptr(), (int)T, (int)H, (int)G, (int)D, (int)Dv,
                           (int)page, PB, (float)scale, (int)window, PB ? (int)pool : 0, f32(q), nsplit,
-                          nsplit > 1 ? part.data_ptr<float>() : nullptr, stream()), "sm_attention");
+                          nsplit > 1 ? part.data_ptr<float>() : nullptr, (int)kld, (int)vld, stream()), "sm_attention");
   return out;
 }
 
@@ -334,6 +369,248 @@ at::Tensor sm_ssd_scan(const at::Tensor& xbc, const at::Tensor& u, int64_t dt0, 
   return y;
 }
 
+// ---------------------------------------------------------------------------------- post-norm layers
+void chk_act2(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.is_contiguous() && is_act(t), name, ": contiguous fp32 / bf16 [rows, cols]");
+}
+
+at::Tensor sm_embed_bigram(const at::Tensor& ids, const at::Tensor& table, const at::Tensor& bigram, at::Tensor& prev_tok,
+                           const at::Tensor& tok_seq, const at::Tensor& tok_pos, const at::Tensor& seq_slot,
+                           const at::Tensor& seq_start, const at::Tensor& seq_len, const at::Tensor& seq_off, int64_t n,
+                           int64_t buckets, int64_t mul_prev, int64_t mul_cur) {
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kLong && ids.is_contiguous() && ids.dim() == 1, "ids: int64 [T]");
+  chk_act2(table, "table");
+  chk_act2(bigram, "bigram");
+  TORCH_CHECK(bigram.scalar_type() == table.scalar_type() && bigram.size(1) == table.size(1) && bigram.size(0) == buckets + 1,
+              "bigram: [buckets + 1, W]");
+  TORCH_CHECK(prev_tok.is_cuda() && prev_tok.scalar_type() == at::kLong && prev_tok.is_contiguous(), "prev_tok: int64 [slots]");
+  for (const at::Tensor* t : {&tok_seq, &tok_pos, &seq_slot, &seq_start, &seq_len, &seq_off}) chk_i32(*t, "metadata");
+  const int64_t T = ids.size(0);
+  TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T && seq_slot.numel() >= n && seq_start.numel() >= n &&
+                  seq_len.numel() >= n && seq_off.numel() >= n, "metadata sizes");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(table.device());
+  auto out = at::empty({T, table.size(1)}, table.options().dtype(at::kFloat));
+  check(edge_sm_embed_bigram(ids.data_ptr<int64_t>(), table.data_ptr(), bigram.data_ptr(), prev_tok.data_ptr<int64_t>(),
+                             tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(),
+                             seq_start.data_ptr<int>(), seq_len.data_ptr<int>(), seq_off.data_ptr<int>(),
+                             out.data_ptr<float>(), (int)T, (int)n, (int)table.size(1), (int)table.size(0), (long)buckets,
+                             (long)mul_prev, (long)mul_cur, f32(table), stream()), "sm_embed_bigram");
+  return out;
+}
+
+at::Tensor sm_canon(const at::Tensor& x, const at::Tensor& w, at::Tensor& state, const at::Tensor& tok_seq,
+                    const at::Tensor& tok_pos, const at::Tensor& seq_slot, const at::Tensor& seq_start,
+                    const at::Tensor& seq_len, const at::Tensor& seq_off, int64_t n, int64_t max_len, bool out_f32) {
+  chk_f32(x, "x");
+  chk_f32(w, "weight");
+  chk_f32(state, "state");
+  for (const at::Tensor* t : {&tok_seq, &tok_pos, &seq_slot, &seq_start, &seq_len, &seq_off}) chk_i32(*t, "metadata");
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && w.size(0) == x.size(1), "x [T, W], weight [W, taps]");
+  const int64_t T = x.size(0), W = x.size(1), taps = w.size(1);
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == std::max<int64_t>(taps - 1, 1) && state.size(2) == W,
+              "state: fp32 [slots, taps - 1, W]");
+  TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T && seq_slot.numel() >= n, "metadata sizes");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  auto out = at::empty({T, W}, x.options().dtype(act_type(out_f32)));
+  check(edge_sm_canon(x.data_ptr<float>(), (int)W, w.data_ptr<float>(), state.data_ptr<float>(), tok_seq.data_ptr<int>(),
+                      tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(), seq_start.data_ptr<int>(), seq_len.data_ptr<int>(),
+                      seq_off.data_ptr<int>(), out.data_ptr(), (int)T, (int)n, (int)taps, (int)max_len, out_f32, stream()),
+        "sm_canon");
+  return out;
+}
+
+at::Tensor sm_layer_norm(const at::Tensor& x, const at::Tensor& w, const at::Tensor& b, double eps, bool out_f32) {
+  chk_f32(x, "x");
+  chk_f32(w, "weight");
+  chk_f32(b, "bias");
+  TORCH_CHECK(x.dim() == 2 && w.numel() == x.size(1) && b.numel() == x.size(1), "x [T, W], weight / bias [W]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  auto y = at::empty_like(x, x.options().dtype(act_type(out_f32)));
+  check(edge_sm_layer_norm(x.data_ptr<float>(), w.data_ptr<float>(), b.data_ptr<float>(), y.data_ptr(), (int)x.size(0),
+                           (int)x.size(1), (float)eps, out_f32, stream()), "sm_layer_norm");
+  return y;
+}
+
+void sm_ln_residual(at::Tensor& x, const std::optional<at::Tensor>& y, const at::Tensor& w, const at::Tensor& b, double eps,
+                    const std::optional<at::Tensor>& parts, const std::optional<at::Tensor>& part_w) {
+  chk_f32(x, "x");
+  chk_f32(w, "weight");
+  chk_f32(b, "bias");
+  TORCH_CHECK(x.dim() == 2 && w.numel() == x.size(1) && b.numel() == x.size(1), "x [T, W], weight / bias [W]");
+  TORCH_CHECK(y || parts, "nothing to norm");
+  const int64_t T = x.size(0), W = x.size(1);
+  int K = 0, is_f32 = 0;
+  if (y) {
+    chk_act2(*y, "y");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == W, "y: [T, W]");
+    is_f32 = f32(*y);
+  }
+  if (parts) {
+    TORCH_CHECK(part_w, "part weights missing");
+    chk_f32(*part_w, "part weights");
+    TORCH_CHECK(parts->is_cuda() && parts->is_contiguous() && is_act(*parts) && parts->dim() == 3 && parts->size(0) == T &&
+                    parts->size(2) == W && part_w->dim() == 2 && part_w->size(0) == T && part_w->size(1) == parts->size(1) &&
+                    (!y || parts->scalar_type() == y->scalar_type()), "parts [T, K, W], weights fp32 [T, K]");
+    K = (int)parts->size(1);
+    is_f32 = f32(*parts);
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  check(edge_sm_ln_residual(x.data_ptr<float>(), y ? y->data_ptr() : nullptr, parts ? parts->data_ptr() : nullptr,
+                            parts ? part_w->data_ptr<float>() : nullptr, K, w.data_ptr<float>(), b.data_ptr<float>(), (int)T,
+                            (int)W, (float)eps, is_f32, stream()), "sm_ln_residual");
+}
+
+at::Tensor sm_rms_cols(const at::Tensor& u, int64_t c0, int64_t C, const at::Tensor& w, double eps, bool out_f32) {
+  TORCH_CHECK(is_act(u) && (u.scalar_type() == at::kFloat) == out_f32, "u: fp32 / bf16, output of the same type");
+  const int ld = row_ld(u, "u");
+  chk_f32(w, "weight");
+  TORCH_CHECK(c0 >= 0 && C > 0 && c0 + C <= u.size(1) && w.numel() == C, "columns out of range / weight [C]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(u.device());
+  auto y = at::empty({u.size(0), C}, u.options());
+  check(edge_sm_rms_cols(u.data_ptr(), ld, (int)c0, (int)C, w.data_ptr<float>(), y.data_ptr(), (int)u.size(0), (float)eps,
+                         f32(u), stream()), "sm_rms_cols");
+  return y;
+}
+
+at::Tensor sm_head_norm_gate(const at::Tensor& y, const at::Tensor& z, const at::Tensor& w, int64_t heads, double eps,
+                             bool out_f32) {
+  chk_f32(y, "y");
+  chk_f32(w, "weight");
+  const int z_ld = row_ld(z, "z");
+  TORCH_CHECK(y.dim() == 2 && heads > 0 && y.size(1) % heads == 0 && w.numel() == y.size(1) / heads && is_act(z) &&
+                  z.size(0) == y.size(0) && z.size(1) == y.size(1) && (z.scalar_type() == at::kFloat) == out_f32,
+              "y fp32 [T, heads P], z [T, heads P], weight [P]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(y.device());
+  auto out = at::empty({y.size(0), y.size(1)}, z.options());
+  check(edge_sm_head_norm_gate(y.data_ptr<float>(), z.data_ptr(), z_ld, w.data_ptr<float>(), out.data_ptr(), (int)y.size(0),
+                               (int)heads, (int)(y.size(1) / heads), (float)eps, f32(z), stream()), "sm_head_norm_gate");
+  return out;
+}
+
+at::Tensor sm_glu_clamp(const at::Tensor& u, int64_t ff, double limit) {
+  TORCH_CHECK(is_act(u), "u: fp32 / bf16");
+  const int ld = row_ld(u, "u");
+  TORCH_CHECK(ff >= 0 && 2 * ff <= u.size(1), "u: [T, gate | up]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(u.device());
+  auto y = at::empty({u.size(0), ff}, u.options());
+  check(edge_sm_glu_clamp(u.data_ptr(), ld, y.data_ptr(), (int)u.size(0), (int)ff, (float)limit, f32(u), stream()),
+        "sm_glu_clamp");
+  return y;
+}
+
+at::Tensor sm_latent_write(const std::optional<at::Tensor>& u, int64_t c0, const std::optional<at::Tensor>& w, double eps,
+                           const at::Tensor& q, const at::Tensor& q_lat, const at::Tensor& tok_seq, const at::Tensor& tok_pos,
+                           const at::Tensor& seq_slot, const at::Tensor& ptab, const std::optional<at::Tensor>& cs,
+                           at::Tensor& pages, int64_t kvr, int64_t rot) {
+  chk_i32(tok_seq, "tok_seq");
+  chk_i32(tok_pos, "tok_pos");
+  chk_i32(seq_slot, "seq_slot");
+  chk_table(ptab);
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() && is_act(q), "q: [T, H, D + R]");
+  TORCH_CHECK(pages.is_cuda() && pages.is_contiguous() && pages.dim() == 4 && pages.size(2) == 1 &&
+                  pages.scalar_type() == q.scalar_type() && pages.size(3) > kvr, "pages: [pages, page, 1, kv_rank + R]");
+  const int64_t T = q.size(0), H = q.size(1), R = pages.size(3) - kvr, D = q.size(2) - R, page = pages.size(1);
+  TORCH_CHECK(D >= 0 && q_lat.is_cuda() && q_lat.dim() == 3 && q_lat.size(0) == T && q_lat.size(1) == H &&
+                  q_lat.size(2) == kvr && q_lat.stride(2) == 1 && q_lat.scalar_type() == q.scalar_type(),
+              "q_lat: [T, H, kv_rank], rows contiguous");
+  TORCH_CHECK(tok_seq.numel() == T && tok_pos.numel() == T, "metadata sizes");
+  int ld = 0;
+  if (u) {
+    ld = row_ld(*u, "u");
+    TORCH_CHECK(w, "latent norm weight missing");
+    chk_f32(*w, "latent norm weight");
+    TORCH_CHECK(u->scalar_type() == q.scalar_type() && u->size(0) == T && c0 >= 0 && c0 + kvr + R <= u->size(1) &&
+                    w->numel() == kvr, "u: [T, .. latent | key part ..]");
+  }
+  if (rot > 0) {
+    TORCH_CHECK(cs, "rotary table missing");
+    chk_f32(*cs, "rotary table");
+    TORCH_CHECK(cs->dim() == 3 && cs->size(1) == rot / 2 && cs->size(2) == 2, "rotary table: [positions, rot / 2, 2]");
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  auto qc = at::empty({T, H, kvr + R}, q.options());
+  check(edge_sm_latent_write(u ? u->data_ptr() : nullptr, ld, (int)c0, u ? w->data_ptr<float>() : nullptr, (float)eps,
+                             q.data_ptr(), q_lat.data_ptr(), (long)q_lat.stride(0), (long)q_lat.stride(1),
+                             tok_seq.data_ptr<int>(), tok_pos.data_ptr<int>(), seq_slot.data_ptr<int>(), ptab.data_ptr<int>(),
+                             (int)ptab.stride(0), rot > 0 ? cs->data_ptr<float>() : nullptr, pages.data_ptr(), qc.data_ptr(),
+                             (int)T, (int)H, (int)D, (int)R, (int)kvr, (int)rot, (int)page, f32(q), stream()),
+        "sm_latent_write");
+  return qc;
+}
+
+at::Tensor sm_delta_prep(const at::Tensor& qkv, const at::Tensor& u, int64_t b0, const at::Tensor& a, const at::Tensor& dt_bias,
+                         const at::Tensor& A_log, int64_t H, int64_t G, int64_t N) {
+  chk_act2(qkv, "qkv");
+  const int ld = row_ld(u, "u");
+  chk_f32(a, "a");
+  chk_f32(dt_bias, "dt_bias");
+  chk_f32(A_log, "A_log");
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(u.scalar_type() == qkv.scalar_type() && u.size(0) == T && b0 >= 0 && b0 + H <= u.size(1) &&
+                  qkv.size(1) >= 2 * G * N && a.dim() == 2 && a.size(0) == T && a.size(1) == H * N &&
+                  dt_bias.numel() == H * N && A_log.numel() == H, "delta prep shapes");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(qkv.device());
+  auto prep = at::empty({T, 2 * G * N + H * N + H}, qkv.options().dtype(at::kFloat));
+  check(edge_sm_delta_prep(qkv.data_ptr(), (int)qkv.size(1), u.data_ptr(), ld, (int)b0, a.data_ptr<float>(),
+                           dt_bias.data_ptr<float>(), A_log.data_ptr<float>(), prep.data_ptr<float>(), (int)T, (int)H,
+                           (int)G, (int)N, f32(qkv), stream()), "sm_delta_prep");
+  return prep;
+}
+
+at::Tensor sm_delta_scan(const at::Tensor& prep, const at::Tensor& qkv, at::Tensor& state, const at::Tensor& seq_slot,
+                         const at::Tensor& seq_start, const at::Tensor& seq_len, const at::Tensor& seq_off, int64_t n,
+                         int64_t H, int64_t G, int64_t N, int64_t P) {
+  chk_f32(prep, "prep");
+  chk_f32(state, "state");
+  chk_act2(qkv, "qkv");
+  for (const at::Tensor* t : {&seq_slot, &seq_start, &seq_len, &seq_off}) chk_i32(*t, "metadata");
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(prep.dim() == 2 && prep.size(0) == T && prep.size(1) == 2 * G * N + H * N + H &&
+                  qkv.size(1) == 2 * G * N + H * P, "prep [T, q | k | decay | beta], qkv [T, q | k | v]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == N && state.size(3) == P,
+              "state: fp32 [slots, heads, N, P]");
+  TORCH_CHECK(seq_slot.numel() >= n && seq_start.numel() >= n && seq_len.numel() >= n && seq_off.numel() >= n,
+              "sequence metadata: [n]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(qkv.device());
+  auto y = at::empty({T, H * P}, prep.options());
+  check(edge_sm_delta_scan(prep.data_ptr<float>(), (int)prep.size(1), qkv.data_ptr(), (int)qkv.size(1), state.data_ptr<float>(),
+                           seq_slot.data_ptr<int>(), seq_start.data_ptr<int>(), seq_len.data_ptr<int>(),
+                           seq_off.data_ptr<int>(), y.data_ptr<float>(), (int)n, (int)H, (int)G, (int)N, (int)P, f32(qkv),
+                           stream()), "sm_delta_scan");
+  return y;
+}
+
+std::tuple<at::Tensor, at::Tensor> sm_moe_route(const at::Tensor& h, const at::Tensor& router, int64_t top, double scale) {
+  chk_act2(h, "h");
+  chk_f32(router, "router");
+  TORCH_CHECK(router.dim() == 2 && router.size(1) == h.size(1), "router: fp32 [E, W]");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(h.device());
+  auto idx = at::empty({h.size(0), top}, h.options().dtype(at::kInt));
+  auto wts = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
+  check(edge_sm_moe_route(h.data_ptr(), (int)h.size(1), router.data_ptr<float>(), (int)router.size(0), (int)top, (float)scale,
+                          idx.data_ptr<int>(), wts.data_ptr<float>(), (int)h.size(0), f32(h), stream()), "sm_moe_route");
+  return {idx, wts};
+}
+
+at::Tensor sm_moe_experts(const at::Tensor& h, const at::Tensor& idx, const at::Tensor& w_gu, const at::Tensor& w_down,
+                          double limit) {
+  chk_act2(h, "h");
+  chk_i32(idx, "idx");
+  const int64_t T = h.size(0), W = h.size(1);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == T, "idx: int32 [T, top]");
+  TORCH_CHECK(w_gu.is_cuda() && w_gu.is_contiguous() && w_gu.dim() == 3 && w_gu.size(2) == W && w_gu.size(1) % 2 == 0 &&
+                  w_down.is_cuda() && w_down.is_contiguous() && w_down.dim() == 3 && w_down.size(0) == w_gu.size(0) &&
+                  w_down.size(1) == W && w_down.size(2) == w_gu.size(1) / 2 && w_gu.scalar_type() == h.scalar_type() &&
+                  w_down.scalar_type() == h.scalar_type(), "experts: w_gu [E, 2 ff, W], w_down [E, W, ff]");
+  const int64_t top = idx.size(1), ff = w_gu.size(1) / 2;
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(h.device());
+  auto y = at::empty({T * top, ff}, h.options());
+  auto out = at::empty({T, top, W}, h.options());
+  check(edge_sm_moe_experts(h.data_ptr(), (int)W, idx.data_ptr<int>(), (int)top, w_gu.data_ptr(), w_down.data_ptr(), (int)ff,
+                            (float)limit, y.data_ptr(), out.data_ptr(), (int)T, f32(h), stream()), "sm_moe_experts");
+  return out;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -348,4 +625,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("sm_attention", &sm_attention);
   m.def("sm_conv_silu", &sm_conv_silu);
   m.def("sm_ssd_scan", &sm_ssd_scan);
+  m.def("sm_embed_bigram", &sm_embed_bigram);
+  m.def("sm_canon", &sm_canon);
+  m.def("sm_layer_norm", &sm_layer_norm);
+  m.def("sm_ln_residual", &sm_ln_residual);
+  m.def("sm_rms_cols", &sm_rms_cols);
+  m.def("sm_head_norm_gate", &sm_head_norm_gate);
+  m.def("sm_glu_clamp", &sm_glu_clamp);
+  m.def("sm_latent_write", &sm_latent_write);
+  m.def("sm_delta_prep", &sm_delta_prep);
+  m.def("sm_delta_scan", &sm_delta_scan);
+  m.def("sm_moe_route", &sm_moe_route);
+  m.def("sm_moe_experts", &sm_moe_experts);
 }

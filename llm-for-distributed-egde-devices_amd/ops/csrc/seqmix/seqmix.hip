@@ -10,38 +10,9 @@
 // walked in the same order from the same first key, each block mean sums its rows in position
 // order, and the recurrence steps token by token.
 #include "common.h"
+#include "seqmix/seqmix_common.h"
 
 namespace {
-
-template <typename T> __device__ __forceinline__ float ldf(const T* p);
-template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
-template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p) { return bf2f(*p); }
-template <typename T> __device__ __forceinline__ void stf(T* p, float v);
-template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
-template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
-
-template <typename KT> __device__ __forceinline__ void load8(const KT* p, float* f);
-template <> __device__ __forceinline__ void load8<float>(const float* p, float* f) {
-  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
-  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
-}
-template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float* f) {
-  unpack8(*reinterpret_cast<const uint4*>(p), f);
-}
-
-template <typename T> __device__ __forceinline__ void store8(T* p, const float* f);
-template <> __device__ __forceinline__ void store8<float>(float* p, const float* f) {
-  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
-  *reinterpret_cast<float4*>(p + 4) = make_float4(f[4], f[5], f[6], f[7]);
-}
-template <> __device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float* f) {
-  *reinterpret_cast<uint4*>(p) = pack8(f);
-}
-
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
-__device__ __forceinline__ float siluf_(float x) { return x * sigmoidf_(x); }
-
-constexpr int NT = 256;
 
 // ---------------------------------------------------------------------------------- rows
 template <typename T>
@@ -231,7 +202,7 @@ constexpr int KC = 256;
 
 template <typename KT, int RMAX, int DVL, bool VEC>
 __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const KT* __restrict__ vbase, int cnt, int g,
-                                           int G, int D, int Dv, int R, const float* q_s, float* s_s, int* row_s,
+                                           int kld, int vld, int D, int Dv, int R, const float* q_s, float* s_s, int* row_s,
                                            float* m_s, float* l_s, float* a_s, int rowidx, float (&acc)[RMAX][VEC ? 8 : DVL]) {
   constexpr int AW = VEC ? 8 : DVL;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -241,7 +212,7 @@ __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const K
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) a[r] = 0.f;
     if (tid < cnt) {
-      const KT* kr = kbase + ((size_t)rowidx * G + g) * D;
+      const KT* kr = kbase + (size_t)rowidx * kld + g * D;
       if constexpr (VEC) {                                  // rows are 16-byte aligned: D % 8 == 0
         for (int d = 0; d < D; d += 8) {
           float kv[8];
@@ -309,7 +280,7 @@ __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const K
 #pragma unroll
       for (int k = 0; k < UN; ++k) {
         const int jk = j + k * KPR + ksub;
-        if (live && jk < j1) load8<KT>(vbase + ((size_t)row_s[jk] * G + g) * Dv + dpart * 8, vv[k]);
+        if (live && jk < j1) load8<KT>(vbase + (size_t)row_s[jk] * vld + g * Dv + dpart * 8, vv[k]);
         else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) vv[k][e] = 0.f;
@@ -331,7 +302,7 @@ __device__ __forceinline__ void attn_chunk(const KT* __restrict__ kbase, const K
       float vv[UN][DVL];
 #pragma unroll
       for (int k = 0; k < UN; ++k) {
-        const KT* vr = vbase + ((size_t)row_s[min(j + k, j1 - 1)] * G + g) * Dv;
+        const KT* vr = vbase + (size_t)row_s[min(j + k, j1 - 1)] * vld + g * Dv;
 #pragma unroll
         for (int dl = 0; dl < DVL; ++dl) vv[k][dl] = lane + 64 * dl < Dv ? ldf<KT>(vr + lane + 64 * dl) : 0.f;
       }
@@ -359,7 +330,9 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
                                                   const int* __restrict__ seq_slot, const int* __restrict__ ptab,
                                                   int ptab_ld, T* __restrict__ out, int H, int G, int D, int Dv,
                                                   int page, int PB, float scale, int window, int pool, int nsp, int nsplit,
-                                                  float* __restrict__ part) {
+                                                  float* __restrict__ part, int kld, int vld) {
+  // kld / vld: elements between consecutive cached rows of kp / vp (G * D and G * Dv for separate key
+  // and value pages; a latent cache whose value is a slice of the key row passes the same stride twice)
   extern __shared__ __attribute__((aligned(16))) float smem[];
   // more than RMAX query heads per kv head: nsp workgroups share the kv head, RMAX heads each
   const int t = blockIdx.x, g = blockIdx.y / nsp, r0 = (blockIdx.y % nsp) * RMAX;
@@ -398,13 +371,13 @@ __global__ void __launch_bounds__(NT) attn_kernel(const T* __restrict__ q, const
     if (ci < ci0 || ci >= ci1) continue;
     const int j = jlo + c0 + tid;
     const int rowidx = c0 + tid < nt ? pt[j / page] * page + j % page : 0;
-    attn_chunk<T, RMAX, DVL, VEC>(kp, vp, min(KC, nt - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
+    attn_chunk<T, RMAX, DVL, VEC>(kp, vp, min(KC, nt - c0), g, kld, vld, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
   }
   for (int c0 = 0; c0 < nb; c0 += KC, ++ci) {
     if (ci < ci0 || ci >= ci1) continue;
     const int p0 = (c0 + tid) * pool;
     const int rowidx = c0 + tid < nb ? pt[p0 / page] * PB + (p0 % page) / pool : 0;
-    attn_chunk<float, RMAX, DVL, VEC>(kb, vb, min(KC, nb - c0), g, G, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
+    attn_chunk<float, RMAX, DVL, VEC>(kb, vb, min(KC, nb - c0), g, G * D, G * Dv, D, Dv, R, q_s, s_s, row_s, m_s, l_s, a_s, rowidx, acc);
   }
   // sum the four waves' partial outputs, normalise, gate
   if constexpr (VEC) {                                       // add up the lanes that walked different keys
@@ -495,7 +468,7 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
     const bf16_t* __restrict__ vp, const float* __restrict__ kb, const float* __restrict__ vb,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_start, const int* __restrict__ seq_len,
     const int* __restrict__ seq_off, const int* __restrict__ ptab, int ptab_ld, bf16_t* __restrict__ out, int n, int H,
-    int G, int PB, float scale_log2, int window, int pool) {
+    int G, int PB, float scale_log2, int window, int pool, int kld, int vld) {
   constexpr int D = 32 * DK, Dv = 16 * DV;
   constexpr int KS = D * 2 + 16, VS = Dv * 2 + 16, PS = MK * 2 + 16;      // LDS row strides in bytes
   __shared__ __attribute__((aligned(16))) char k_lds[MK * KS];
@@ -560,8 +533,8 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
       const int r = e / cpr, c = e % cpr;
       uint4 v = make_uint4(0, 0, 0, 0);
       if (tok) {
-        v = isk ? *reinterpret_cast<const uint4*>(kp + ((prow + r) * G + g) * D + c * 8)
-                : *reinterpret_cast<const uint4*>(vp + ((prow + r) * G + g) * Dv + c * 8);
+        v = isk ? *reinterpret_cast<const uint4*>(kp + (prow + r) * kld + g * D + c * 8)
+                : *reinterpret_cast<const uint4*>(vp + (prow + r) * vld + g * Dv + c * 8);
       } else if (base + r < nbmax) {
         const int p0 = (base + r) * pool;
         const size_t row = ((size_t)page_of(p0 / MK) * PB + (p0 % MK) / pool) * G + g;
@@ -1148,29 +1121,42 @@ int edge_sm_pool_blocks(const void* kp, const void* vp, float* kb, float* vb, co
 
 // nsplit > 1: the keys of every query are walked by nsplit workgroups (decode steps: few queries, long
 // windows); part = fp32 scratch [rows, G * nsp, nsplit, rmax * (Dv + 2)] (edge_sm_attention_part_floats)
-size_t edge_sm_attention_part_floats(int rows, int H, int G, int Dv, int nsplit) {
-  const int R = H / G, rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16, nsp = (R + rmax - 1) / rmax;
+static size_t attn_lds_bytes(int rmax, int D, int Dv) {
+  return sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 3 * rmax) + sizeof(int) * KC;
+}
+
+// query heads of one kv head that share a workgroup: the whole group up to 16, fewer while their rows
+// (queries, scores, partial outputs) would not fit 64 KB of LDS; 0: not even one head fits
+int edge_sm_attention_rmax(int H, int G, int D, int Dv) {
+  const int R = H / G;
+  int rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16;
+  while (rmax > 1 && attn_lds_bytes(rmax, D, Dv) > 64 * 1024) rmax >>= 1;
+  return attn_lds_bytes(rmax, D, Dv) > 64 * 1024 ? 0 : rmax;
+}
+
+size_t edge_sm_attention_part_floats(int rows, int H, int G, int D, int Dv, int nsplit) {
+  const int R = H / G, rmax = max(1, edge_sm_attention_rmax(H, G, D, Dv)), nsp = (R + rmax - 1) / rmax;
   return (size_t)rows * G * nsp * nsplit * rmax * (Dv + 2);
 }
 
 int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* kp, const void* vp, const float* kb,
                       const float* vb, const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* ptab,
                       int ptab_ld, void* out, int rows, int H, int G, int D, int Dv, int page, int PB, float scale,
-                      int window, int pool, int f32, int nsplit, float* part, hipStream_t st) {
+                      int window, int pool, int f32, int nsplit, float* part, int kld, int vld, hipStream_t st) {
   if (rows == 0) return 0;
-  if (G <= 0 || H % G || Dv > 256) return -2;
+  if (G <= 0 || H % G || Dv > 512) return -2;
   const int R = H / G;
-  const int rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16;
+  const int rmax = edge_sm_attention_rmax(H, G, D, Dv);
+  if (rmax == 0) return -3;
   const int nsp = (R + rmax - 1) / rmax;
   if (nsplit < 1 || (nsplit > 1 && !part)) return -2;
-  const size_t lds = sizeof(float) * ((size_t)rmax * D + (size_t)rmax * KC + (size_t)rmax * Dv + 3 * rmax) +
-                     sizeof(int) * KC;
-  if (lds > 64 * 1024) return -3;
-  const bool vec = D % 8 == 0 && Dv % 8 == 0;
+  const size_t lds = attn_lds_bytes(rmax, D, Dv);
+  const bool vec = D % 8 == 0 && Dv % 8 == 0 && kld % 8 == 0 && vld % 8 == 0;
 #define SM_ATT_V(RM, DL, V)                                                                                         \
   SM_T(f32, hipLaunchKernelGGL((attn_kernel<T, RM, DL, V>), dim3(rows, G * nsp, nsplit), dim3(NT), lds, st, (const T*)q,         \
                                (const T*)gate, gate_ld, (const T*)kp, (const T*)vp, kb, vb, tok_seq, tok_pos,       \
-                               seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool, nsp, nsplit, part))
+                               seq_slot, ptab, ptab_ld, (T*)out, H, G, D, Dv, page, PB, scale, window, pool, nsp, nsplit, part, \
+                               kld, vld))
 #define SM_ATT(RM, DL)               \
   do {                               \
     if (vec) SM_ATT_V(RM, DL, true); \
@@ -1186,7 +1172,8 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
   }
   if (Dv <= 64) { SM_ATT_R(1); }
   else if (Dv <= 128) { SM_ATT_R(2); }
-  else { SM_ATT_R(4); }
+  else if (Dv <= 256) { SM_ATT_R(4); }
+  else { SM_ATT_R(8); }
 #undef SM_ATT_R
 #undef SM_ATT
 #undef SM_ATT_V
@@ -1263,8 +1250,8 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
                            const float* kb, const float* vb, const int* seq_slot, const int* seq_start,
                            const int* seq_len, const int* seq_off, const int* ptab, int ptab_ld, void* out, int n,
                            int qtiles, int H, int G, int D, int Dv, int page, int PB, float scale, int window,
-                           int pool, hipStream_t st) {
-  if (page != MK || G <= 0 || H % G) return 1;
+                           int pool, int kld, int vld, hipStream_t st) {
+  if (page != MK || G <= 0 || H % G || kld % 8 || vld % 8) return 1;
   if (n == 0 || qtiles == 0) return 0;
   const float sl2 = scale * 1.4426950408889634f;
   // query heads per workgroup: a staged tile can serve 4 or 2 heads of a kv group, but the kernel is
@@ -1278,7 +1265,7 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
 #define SM_MF_R(DK, DV, RH)                                                                                        \
   hipLaunchKernelGGL((attn_mfma_kernel<DK, DV, RH>), dim3(qtiles, H / RH), dim3(NT), 0, st, (const bf16_t*)q,     \
                      (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb, seq_slot,         \
-                     seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window, pool)
+                     seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window, pool, kld, vld)
 #define SM_MF(DK, DV)                      \
   do {                                     \
     if (rh == 4) SM_MF_R(DK, DV, 4);       \
@@ -1291,6 +1278,9 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
   else if (D == 128 && Dv == 64) SM_MF(4, 4);
   else if (D == 64 && Dv == 128) SM_MF(2, 8);
   else if (D == 32 && Dv == 32) SM_MF(1, 2);
+  else if (D == 128 && Dv == 96) SM_MF(4, 6);                // latent rows: latent + shared key part, value = the latent
+  else if (D == 160 && Dv == 128) SM_MF(5, 8);
+  else if (D == 192 && Dv == 128) SM_MF(6, 8);
   else return 1;
 #undef SM_MF
 #undef SM_MF_R

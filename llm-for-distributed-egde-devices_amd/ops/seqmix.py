@@ -382,7 +382,7 @@ def canon_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, meta:
     taps = weight.shape[1]
     if _gpu(x):
         return _ext().sm_canon(x, weight, state, meta.tok_seq, meta.tok_pos, meta.seq_slot, meta.seq_start, meta.seq_len,
-                               meta.seq_off, int(meta.n), out_dtype == torch.float32)
+                               meta.seq_off, int(meta.n), int(meta.max_len), out_dtype == torch.float32)
     out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
     W = x.shape[1]
     for slot, start, n, off in meta.host:
