@@ -48,15 +48,15 @@ class PagedCache:
         for r, s in enumerate(run_specs):
             rc = RunCache()
             latent, delta = getattr(s, "latent", None), getattr(s, "delta", None)
-            if latent is not None or delta is not None:
+            if getattr(s, "attn", None) is None:             # a post-norm layer: one mixer of either kind
                 if latent is not None:
                     src = s.latent.kv_from
                     if src is None:
                         rc.lat = torch.zeros(num_pages, page, 1, s.latent.cache_dim, dtype=dtype, device=device)
                     else:                                  # the latest earlier run of the named layer
                         rc.lat = self.runs[max(j for j in range(r) if run_layers[j] == src)].lat
-                else:
-                    d = s.delta
+                elif delta is not None:
+                    d = delta
                     rc.conv = torch.zeros(slots, max(d.conv - 1, 1), d.conv_channels, dtype=dtype, device=device)
                     rc.ssm = torch.zeros(slots, d.heads, d.dim, d.vdim, dtype=torch.float32, device=device)
                 if canon_taps:

@@ -193,22 +193,25 @@ def moe(h, w, p: str, m: dict):
 def forward(cfg: dict, w: Dict[str, torch.Tensor], ids: List[int], taps: Optional[list] = None) -> torch.Tensor:
     """Logits [T, vocab] of one sequence; ``taps`` receives the residual stream after every layer."""
     w = {k: v.to(F64) for k, v in w.items()}
+    ids = [int(t) for t in ids]
     eps = float(cfg["norm"]["eps"])
-    x = embed(ids, w["embed"], w["bigram"], cfg["embedding"]["bigram"])
+    big = (cfg.get("embedding") or {}).get("bigram")
+    x = embed(ids, w["embed"], w["bigram"], big) if big else w["embed"][ids]
+    reads = (lambda x, name: input_conv(x, w[name])) if (cfg.get("canon") or {}).get("taps") else (lambda x, name: x)
     kept = {}
     for i, l in enumerate(cfg["layers"]):
         p = f"l{i}."
-        h = input_conv(x, w[p + "canon1"])
+        h = reads(x, p + "canon1")
         if l["type"] == "latent_attention":
             src = l["mixer"].get("kv_from")
             y, kept[i] = latent_attention(h, w, p + "mix.", l["mixer"], eps, kept[src] if src is not None else None)
         elif l["type"] == "channel_delta":
-            y = channel_delta(h, w, p + "mix.", dict(l["mixer"], taps=None), eps)
+            y = channel_delta(h, w, p + "mix.", l["mixer"], eps)
         else:
             raise ValueError(l["type"])
         x = x + layer_norm(y, w[p + "norm1"], w[p + "norm1.b"], eps)
         if l.get("mlp"):
-            h = input_conv(x, w[p + "canon2"])
+            h = reads(x, p + "canon2")
             x = x + layer_norm(moe(h, w, p + "mlp.", l["mlp"]), w[p + "norm2"], w[p + "norm2.b"], eps)
         if taps is not None:
             taps.append(x.clone())
