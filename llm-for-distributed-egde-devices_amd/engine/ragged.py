@@ -70,8 +70,15 @@ class _DecodeGraph:
             self.warm = True
             return eng.model(self.ids, self.meta, eng.cache, self.rows)
         if self.graph is None:
+            # no cyclic garbage collection while the stream captures: a collected engine of an earlier
+            # request frees pinned buffers and graphs, which the runtime refuses during a capture; what
+            # is garbage already goes first
+            import gc
+            gc.collect()
             g = torch.cuda.CUDAGraph()
             torch.cuda.synchronize()
+            gc_was_on = gc.isenabled()
+            gc.disable()
             try:
                 with torch.cuda.graph(g, pool=eng._pool):
                     self.out = eng.model(self.ids, self.meta, eng.cache, self.rows)
@@ -81,6 +88,9 @@ class _DecodeGraph:
                 torch.cuda.synchronize()
                 eng.use_graphs = False
                 return eng.model(self.ids, self.meta, eng.cache, self.rows)
+            finally:
+                if gc_was_on:
+                    gc.enable()
             if eng._pool is None:
                 eng._pool = g.pool()
             self.graph = g

@@ -563,7 +563,7 @@ def test_decode_graph_replays_match_eager(tmp_path):
     cfg = make_config(width=64)
     w = make_weights(cfg, seed=21)
     reqs = {"a": tokens(40, cfg["vocab"], 1), "b": tokens(25, cfg["vocab"], 2), "c": tokens(30, cfg["vocab"], 3)}
-    sched = [[("a", 9), ("b", 4)]] + [[("a", 1), ("b", 1)]] * 12 + [[("a", 1), ("b", 1), ("c", 11)]] + \
+    sched = [[("a", 10), ("b", 4)]] + [[("a", 1), ("b", 1)]] * 12 + [[("a", 1), ("b", 1), ("c", 11)]] + \
         [[("a", 1), ("b", 1), ("c", 1)]] * 8 + [[("a", 1), ("c", 1)]] * 9 + [[("c", 1)]] * 2
     outs = {}
     for graphs in (False, True):
