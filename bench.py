@@ -102,6 +102,9 @@ def parse(argv=None):
     ap.add_argument("--hybrid-compare", action="store_true",
                     help="instead of the headline workload: prefill / decode throughput of the Nudadra layer-spec "
                          "model beside the parallel-residual decoder of equal size (one JSON line)")
+    ap.add_argument("--hybrid-family", default="nudadra", choices=["nudadra", "pagonex"],
+                    help="with --hybrid-compare: nudadra (beside the parallel-residual decoder) or pagonex (latent "
+                         "attention + gated delta rule + mixture of experts, beside the Nudadra hybrid)")
     ap.add_argument("--hybrid-sizes", default="w1024,w2048", help="comma list of w1024 | w2048 | w4096")
     ap.add_argument("--hybrid-prompt", type=int, default=4096)
     ap.add_argument("--hybrid-batch", type=int, default=4)
@@ -438,7 +441,7 @@ def main(argv=None):
     if args.hybrid_compare:
         from edgellm.engine import ragged_bench
         out = ragged_bench.run(args.hybrid_sizes.split(","), args.hybrid_prompt, args.hybrid_batch, args.steps,
-                               args.device)
+                               args.device, family=args.hybrid_family)
         print(json.dumps(out), flush=True)
         return out
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:

@@ -1,5 +1,8 @@
-"""Prefill / decode throughput of a layer-spec (Nudadra) model beside the closest row-cache model
-of equal size (``bench.py --hybrid-compare``).
+"""Prefill / decode throughput of a layer-spec model beside the closest existing model of equal size
+(``bench.py --hybrid-compare``): the Nudadra hybrid beside the parallel-residual row-cache decoder,
+or (``--hybrid-family pagonex``) the Pagonex model (latent attention and gated delta-rule layers,
+mixture-of-experts feed-forwards) beside the Nudadra hybrid, its closest relative: the same engine,
+windowed attention over the paged cache, a recurrent mixer and a feed-forward per layer.
 
 Sizes resemble real layers (random weights): the hybrid layer has windowed attention with pooled
 blocks + a Mamba-2 mixer + a squared-ReLU feed-forward; the comparison model is the
@@ -18,7 +21,8 @@ from typing import Dict, List
 
 import torch
 
-from ..models.configs import LayerSpec, ModelConfig, SSDSpec, WindowAttnSpec, PRESETS
+from ..models.configs import (DeltaSpec, LatentAttnSpec, LayerSpec, ModelConfig, MoESpec, SSDSpec, WindowAttnSpec,
+                              PRESETS)
 from ..models.decoder import build_model
 from ..models.hybrid import build_hybrid
 from .generate import Generator, SamplingParams
@@ -46,6 +50,38 @@ def hybrid_config(s: dict) -> ModelConfig:
                        embed_scale=1.0)
 
 
+# Pagonex sizes: per layer pair one latent-attention layer (the second reads the first one's cache) and one
+# delta-rule layer; the experts' active width (top x ff + shared) equals the dense feed-forward of the
+# Nudadra size of the same name
+PAGONEX_SIZES = {
+    "w1024": dict(width=1024, layers=4, heads=16, dim=64, rot=32, vdim=64, q_rank=384, kv_rank=128, window=512,
+                  d_heads=16, d_dim=64, d_vdim=64, experts=16, top=3, ff=1024, shared=1024, vocab=32000),
+    "w2048": dict(width=2048, layers=4, heads=16, dim=128, rot=64, vdim=128, q_rank=768, kv_rank=256, window=1024,
+                  d_heads=16, d_dim=128, d_vdim=128, experts=32, top=3, ff=2048, shared=2048, vocab=32000),
+}
+
+
+def pagonex_config(s: dict) -> ModelConfig:
+    yarn = {"rope_type": "yarn", "factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    moe = MoESpec(s["experts"], s["top"], 2.5, s["ff"], 7.0, s["shared"], 7.0)
+    specs = []
+    for i in range(s["layers"]):
+        if i % 2 == 0:
+            a = LatentAttnSpec(s["heads"], s["dim"], s["rot"], s["vdim"], s["q_rank"], s["kv_rank"],
+                               (s["dim"] + s["rot"]) ** -0.5, s["window"], s["rot"], 500000.0, yarn,
+                               kv_from=0 if i else None)
+            specs.append(LayerSpec("latent_attention", latent=a, moe=moe))
+        else:
+            d = DeltaSpec(s["d_heads"], s["d_heads"], s["d_dim"], s["d_vdim"], 4, max(16, s["width"] // 32),
+                          max(16, s["width"] // 32))
+            specs.append(LayerSpec("channel_delta", delta=d, moe=moe))
+    return ModelConfig(arch="pagonex", vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
+                       num_heads=s["heads"], num_kv_heads=1, intermediate_size=0, head_dim=1,
+                       max_position_embeddings=1 << 20, norm="layer", norm_eps=1e-6, act="glu_clamp", name="pagonex-bench",
+                       layer_specs=specs, canon_taps=3, bigram={"buckets": 8191, "mul_prev": 31, "mul_cur": 7},
+                       logit_scale=0.5)
+
+
 def closest_config(s: dict) -> ModelConfig:
     return PRESETS["phi-2"].replace(vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
                                     num_heads=s["heads"], num_kv_heads=s["kv"], head_dim=s["dim"], rotary_dim=s["dim"],
@@ -63,8 +99,8 @@ def _timed(fn, reps: int, warm: int = 1) -> float:
     return (time.perf_counter() - t0) / reps
 
 
-def bench_hybrid(s: dict, prompt: int, batch: int, steps: int, device) -> Dict:
-    model = build_hybrid(hybrid_config(s), torch.bfloat16, device, seed=0)
+def bench_hybrid(s: dict, prompt: int, batch: int, steps: int, device, cfg: ModelConfig = None) -> Dict:
+    model = build_hybrid(cfg if cfg is not None else hybrid_config(s), torch.bfloat16, device, seed=0)
     ids = torch.randint(0, s["vocab"], (prompt,), generator=torch.Generator().manual_seed(0)).tolist()
     page = 64
     eng = RaggedEngine(model, (batch + 1) * ((prompt + steps + 2 * page) // page) * page, slots=batch + 1)
@@ -92,7 +128,9 @@ def op_times(eng: RaggedEngine, entries, close=()) -> Dict[str, float]:
     import torch.nn.functional as F
     marks: List[tuple] = []
     names = ["embedding_scaled", "scalar_rms_norm", "relu2", "cat_cast", "combine_residual", "gated_group_norm",
-             "rope_paged_write", "pool_blocks", "window_pool_attention", "conv_silu", "ssd_scan", "linear_f32"]
+             "rope_paged_write", "pool_blocks", "window_pool_attention", "conv_silu", "ssd_scan", "linear_f32",
+             "embedding_bigram", "canon_conv", "layer_norm_rows", "layer_norm_residual", "rms_norm_cols", "glu_clamp",
+             "latent_write", "delta_prepare", "delta_rule_scan", "head_norm_gate", "moe_route", "moe_experts"]
     saved = {n: getattr(seqmix, n) for n in names}
     lin = F.linear
 
@@ -114,12 +152,15 @@ def op_times(eng: RaggedEngine, entries, close=()) -> Dict[str, float]:
         from ..models import layers as L
         orig_fwd = L.Linear.forward
         L.Linear.forward = wrap("projections", orig_fwd)
+        bmm = torch.bmm
+        torch.bmm = wrap("head_expansions_bmm", bmm)
         eng.step(entries)
         torch.cuda.synchronize()
     finally:
         for n in names:
             setattr(seqmix, n, saved[n])
         L.Linear.forward = orig_fwd
+        torch.bmm = bmm
         if graphs is not None:
             eng.use_graphs = graphs
     for r in close:
@@ -149,8 +190,27 @@ def bench_closest(s: dict, prompt: int, batch: int, steps: int, device) -> Dict:
             "decode_ms_per_step": t_dec * 1e3}
 
 
-def run(sizes: List[str], prompt: int = 4096, batch: int = 4, steps: int = 32, device=None) -> Dict:
+def run_pagonex(sizes: List[str], prompt: int, batch: int, steps: int, device) -> Dict:
+    res = {}
+    r2 = lambda d: {k: (round(v, 2) if isinstance(v, float) else v) for k, v in d.items()}
+    for name in sizes:
+        s = PAGONEX_SIZES[name]
+        p = bench_hybrid(s, prompt, batch, steps, device, pagonex_config(s))
+        torch.cuda.empty_cache()
+        h = bench_hybrid(SIZES[name], prompt, batch, steps, device)
+        torch.cuda.empty_cache()
+        res[name] = {"size": s, "closest_size": SIZES[name], "pagonex": r2(p), "closest_nudadra": r2(h),
+                     "prefill_ratio": round(p["prefill_tok_s"] / h["prefill_tok_s"], 3),
+                     "decode_ratio": round(p["decode_tok_s"] / h["decode_tok_s"], 3)}
+    return {"metric": "prefill / decode tokens/s, Pagonex layer-spec model vs the Nudadra hybrid of equal size",
+            "dtype": "bf16", "data": "synthetic (random weights, random prompt)", "prompt_tokens": prompt,
+            "decode_batch": batch, "decode_steps": steps, "sizes": res}
+
+
+def run(sizes: List[str], prompt: int = 4096, batch: int = 4, steps: int = 32, device=None, family: str = "nudadra") -> Dict:
     device = torch.device(device or "cuda:0")
+    if family == "pagonex":
+        return run_pagonex(sizes, prompt, batch, steps, device)
     res = {}
     for name in sizes:
         s = SIZES[name]

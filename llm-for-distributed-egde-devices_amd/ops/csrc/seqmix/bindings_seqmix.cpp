@@ -70,10 +70,10 @@ int edge_sm_delta_prep(const void* qkv, int Cq, const void* u, int ld, int b0, c
 int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, float* state, const int* seq_slot,
                        const int* seq_start, const int* seq_len, const int* seq_off, float* y, int n, int H, int G, int N,
                        int P, int f32, hipStream_t st);
-int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, int* idx, float* wts, int rows,
-                      int f32, hipStream_t st);
+int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, float* z, int* idx, float* wts,
+                      int rows, int f32, hipStream_t st);
 int edge_sm_moe_experts(const void* h, int W, const int* idx, int top, const void* w_gu, const void* w_down, int ff,
-                        float limit, void* y, void* out, int rows, int f32, hipStream_t st);
+                        float limit, void* y, void* out, int rows, int E, int f32, hipStream_t st);
 }
 
 namespace {
@@ -587,8 +587,10 @@ std::tuple<at::Tensor, at::Tensor> sm_moe_route(const at::Tensor& h, const at::T
   c10::hip::HIPGuardMasqueradingAsCUDA guard(h.device());
   auto idx = at::empty({h.size(0), top}, h.options().dtype(at::kInt));
   auto wts = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
+  auto z = at::empty({h.size(0), router.size(0)}, wts.options());
   check(edge_sm_moe_route(h.data_ptr(), (int)h.size(1), router.data_ptr<float>(), (int)router.size(0), (int)top, (float)scale,
-                          idx.data_ptr<int>(), wts.data_ptr<float>(), (int)h.size(0), f32(h), stream()), "sm_moe_route");
+                          z.data_ptr<float>(), idx.data_ptr<int>(), wts.data_ptr<float>(), (int)h.size(0), f32(h), stream()),
+        "sm_moe_route");
   return {idx, wts};
 }
 
@@ -607,7 +609,8 @@ at::Tensor sm_moe_experts(const at::Tensor& h, const at::Tensor& idx, const at::
   auto y = at::empty({T * top, ff}, h.options());
   auto out = at::empty({T, top, W}, h.options());
   check(edge_sm_moe_experts(h.data_ptr(), (int)W, idx.data_ptr<int>(), (int)top, w_gu.data_ptr(), w_down.data_ptr(), (int)ff,
-                            (float)limit, y.data_ptr(), out.data_ptr(), (int)T, f32(h), stream()), "sm_moe_experts");
+                            (float)limit, y.data_ptr(), out.data_ptr(), (int)T, (int)w_gu.size(0), f32(h), stream()),
+        "sm_moe_experts");
   return out;
 }
 

@@ -242,21 +242,33 @@ __global__ void __launch_bounds__(NT) delta_prep_kernel(const T* __restrict__ qk
   for (int e = tid; e < H; e += NT) pr[2 * GN + HN + e] = sigmoidf_(ldf<T>(u + t * ld + b0 + e));
 }
 
-// One workgroup per (sequence, head, 64 value columns): wave w owns columns 16 w .. 16 w + 15, lane
-// (rg = lane / 16, col = lane % 16) keeps rows rg * NR .. rg * NR + NR - 1 of its column in registers
-// (NR = ceil(N / 4)).  Tokens are staged TC at a time (q, k, decay rows, beta, the 64 values) and
-// stepped in order; the two sums over rows (S^T k and S^T q) are NR FMAs per lane and two cross-lane adds.
+// sum over the 16 lanes of a DPP row (quad swaps, then row rotations by 4 and 8); every lane gets the sum
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xF, 0xF, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xF, 0xF, false));
+  return v;
+}
+
+// One workgroup per (sequence, head, 16 value columns): wave w owns columns 4 w .. 4 w + 3; the 16 lanes of
+// a DPP row share one column, lane rg of the row keeping state rows rg * NR .. rg * NR + NR - 1 in
+// registers (NR = ceil(N / 16) rounded up to 4), so the two sums over rows per token (S^T k and S^T q) are
+// NR FMAs and four in-row DPP adds.  Tokens are staged TC at a time (q, k, decay rows, beta, the 16 values);
+// the next chunk's rows travel global -> registers while the current one is stepped, registers -> the
+// other LDS buffer after it (one barrier per chunk).
 template <typename T, int NR>
 __global__ void __launch_bounds__(NT) delta_scan_kernel(const float* __restrict__ prep, int prep_ld, const T* __restrict__ qkv,
                                                         int Cq, float* __restrict__ state, const int* __restrict__ seq_slot,
                                                         const int* __restrict__ seq_start, const int* __restrict__ seq_len,
                                                         const int* __restrict__ seq_off, float* __restrict__ y, int H, int G,
                                                         int N, int P) {
-  constexpr int TC = NR >= 64 ? 8 : 16, RS = NR + 4, ROW = 4 * RS;   // padded rows: the four row groups hit different banks
-  __shared__ __attribute__((aligned(16))) float q_s[TC][ROW], k_s[TC][ROW], g_s[TC][ROW];
-  __shared__ float v_s[TC][64], b_s[TC];
-  const int s = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * 64, tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6, rg = lane >> 4, col = wave * 16 + (lane & 15), p = p0 + col;
+  constexpr int NP = 16 * NR, TC = NR >= 16 ? 4 : (NR >= 8 ? 8 : 16), EL = TC * 3 * NP / NT;   // EL = 12
+  constexpr int CW = 16;                                     // value columns per workgroup
+  __shared__ __attribute__((aligned(16))) float rows_s[2][TC][3][NP];   // q | k | decay
+  __shared__ float v_s[2][TC][CW], b_s[2][TC];
+  const int s = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * CW, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6, rg = lane & 15, col = wave * 4 + (lane >> 4), p = p0 + col;
   const int start = seq_start[s], len = seq_len[s], off = seq_off[s];
   const int g = h / (H / G), GN = G * N, HN = H * N;
   float* st = state + ((size_t)seq_slot[s] * H + h) * N * P;
@@ -266,50 +278,70 @@ __global__ void __launch_bounds__(NT) delta_scan_kernel(const float* __restrict_
     const int n = rg * NR + i;
     S[i] = (start > 0 && n < N && p < P) ? st[(size_t)n * P + p] : 0.f;
   }
-  for (int t0 = 0; t0 < len; t0 += TC) {
+  float pre[EL], pre_v = 0.f, pre_b = 0.f;
+  auto fetch = [&](int t0) {                                 // rows of tokens t0 .. t0 + TC - 1 into registers
     const int tc = min(TC, len - t0);
-    __syncthreads();
-    for (int e = tid; e < tc * 4 * NR; e += NT) {
-      const int tt = e / (4 * NR), j = e % (4 * NR), n = j, dst = (j / NR) * RS + j % NR;
-      const float* pr = prep + (size_t)(off + t0 + tt) * prep_ld;
-      const bool ok = n < N;
-      q_s[tt][dst] = ok ? pr[g * N + n] : 0.f;
-      k_s[tt][dst] = ok ? pr[GN + g * N + n] : 0.f;
-      g_s[tt][dst] = ok ? pr[2 * GN + h * N + n] : 1.f;
+#pragma unroll
+    for (int i = 0; i < EL; ++i) {
+      const int e = tid + i * NT, tt = e / (3 * NP), r = e % (3 * NP), which = r / NP, n = r % NP;
+      float v = which == 2 ? 1.f : 0.f;                      // rows past N: no decay, no key, no query
+      if (tt < tc && n < N) {
+        const float* pr = prep + (size_t)(off + t0 + tt) * prep_ld;
+        v = which == 0 ? pr[g * N + n] : (which == 1 ? pr[GN + g * N + n] : pr[2 * GN + h * N + n]);
+      }
+      pre[i] = v;
     }
-    for (int e = tid; e < tc * 64; e += NT) {
-      const int tt = e / 64, c = e % 64;
-      v_s[tt][c] = p0 + c < P ? ldf<T>(qkv + (size_t)(off + t0 + tt) * Cq + 2 * GN + h * P + p0 + c) : 0.f;
+    {
+      const int tt = tid / CW, c = tid % CW;
+      pre_v = (tid < TC * CW && tt < tc && p0 + c < P) ? ldf<T>(qkv + (size_t)(off + t0 + tt) * Cq + 2 * GN + h * P + p0 + c) : 0.f;
+      pre_b = tid < tc ? prep[(size_t)(off + t0 + tid) * prep_ld + 2 * GN + HN + h] : 0.f;
     }
-    if (tid < tc) b_s[tid] = prep[(size_t)(off + t0 + tid) * prep_ld + 2 * GN + HN + h];
-    __syncthreads();
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < EL; ++i) {
+      const int e = tid + i * NT;
+      (&rows_s[buf][0][0][0])[e] = pre[i];
+    }
+    if (tid < TC * CW) v_s[buf][tid / CW][tid % CW] = pre_v;
+    if (tid < TC) b_s[buf][tid] = pre_b;
+  };
+  static_assert(TC * CW <= NT && TC * 3 * NP % NT == 0, "staging shape");
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = 0; t0 < len; t0 += TC, buf ^= 1) {
+    const int tc = min(TC, len - t0);
+    const bool more = t0 + TC < len;
+    if (more) fetch(t0 + TC);
     for (int tt = 0; tt < tc; ++tt) {
-      const float4* kq = reinterpret_cast<const float4*>(&k_s[tt][rg * RS]);
-      const float4* gq = reinterpret_cast<const float4*>(&g_s[tt][rg * RS]);
-      const float4* qq = reinterpret_cast<const float4*>(&q_s[tt][rg * RS]);
-      float kv0 = 0.f, kv1 = 0.f;
+      const float4* qq = reinterpret_cast<const float4*>(&rows_s[buf][tt][0][rg * NR]);
+      const float4* kq = reinterpret_cast<const float4*>(&rows_s[buf][tt][1][rg * NR]);
+      const float4* gq = reinterpret_cast<const float4*>(&rows_s[buf][tt][2][rg * NR]);
+      float4 kk[NR / 4];
+      float kv = 0.f;
 #pragma unroll
       for (int i = 0; i < NR / 4; ++i) {
-        const float4 gv = gq[i], kk = kq[i];
+        const float4 gv = gq[i];
+        kk[i] = kq[i];
         S[4 * i] *= gv.x; S[4 * i + 1] *= gv.y; S[4 * i + 2] *= gv.z; S[4 * i + 3] *= gv.w;
-        kv0 += S[4 * i] * kk.x; kv1 += S[4 * i + 1] * kk.y; kv0 += S[4 * i + 2] * kk.z; kv1 += S[4 * i + 3] * kk.w;
+        kv += S[4 * i] * kk[i].x + S[4 * i + 1] * kk[i].y + S[4 * i + 2] * kk[i].z + S[4 * i + 3] * kk[i].w;
       }
-      float kv = kv0 + kv1;
-      kv += __shfl_xor(kv, 16, 64);
-      kv += __shfl_xor(kv, 32, 64);
-      const float w = b_s[tt] * (v_s[tt][col] - kv);
-      float o0 = 0.f, o1 = 0.f;
+      kv = row16_sum(kv);
+      const float w = b_s[buf][tt] * (v_s[buf][tt][col] - kv);
+      float o = 0.f;
 #pragma unroll
       for (int i = 0; i < NR / 4; ++i) {
-        const float4 kk = kq[i], qv = qq[i];
-        S[4 * i] += kk.x * w; S[4 * i + 1] += kk.y * w; S[4 * i + 2] += kk.z * w; S[4 * i + 3] += kk.w * w;
-        o0 += S[4 * i] * qv.x; o1 += S[4 * i + 1] * qv.y; o0 += S[4 * i + 2] * qv.z; o1 += S[4 * i + 3] * qv.w;
+        const float4 qv = qq[i];
+        S[4 * i] += kk[i].x * w; S[4 * i + 1] += kk[i].y * w; S[4 * i + 2] += kk[i].z * w; S[4 * i + 3] += kk[i].w * w;
+        o += S[4 * i] * qv.x + S[4 * i + 1] * qv.y + S[4 * i + 2] * qv.z + S[4 * i + 3] * qv.w;
       }
-      float o = o0 + o1;
-      o += __shfl_xor(o, 16, 64);
-      o += __shfl_xor(o, 32, 64);
+      o = row16_sum(o);
       if (rg == 0 && p < P) y[(size_t)(off + t0 + tt) * H * P + h * P + p] = o;
     }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
   }
   if (p < P) {
 #pragma unroll
@@ -321,24 +353,40 @@ __global__ void __launch_bounds__(NT) delta_scan_kernel(const float* __restrict_
 }
 
 // ---------------------------------------------------------------------------------- mixture of experts
-// One workgroup per token: wave w scores experts w, w + 4, .. (fp32 dot products over the width), the first
-// wave turns the scores into a softmax and picks the `top` largest (lowest index on a tie).
+// Router scores: one wave per (token, expert), fp32 dot product over the width with 8-element loads.
 template <typename T>
-__global__ void __launch_bounds__(NT) moe_route_kernel(const T* __restrict__ h, int W, const float* __restrict__ router, int E,
-                                                       int top, float scale, int* __restrict__ idx, float* __restrict__ wts) {
+__global__ void __launch_bounds__(NT) moe_logits_kernel(const T* __restrict__ h, int W, const float* __restrict__ router,
+                                                        int E, float* __restrict__ z) {
+  const size_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, e = blockIdx.y * (NT / 64) + (threadIdx.x >> 6);
+  if (e >= E) return;
+  const T* hr = h + t * W;
+  const float* rr = router + (size_t)e * W;
+  float acc = 0.f;
+  if (W % 8 == 0) {
+    for (int c = lane * 8; c < W; c += 64 * 8) {
+      float a[8], r[8];
+      load8<T>(hr + c, a);
+      load8<float>(rr + c, r);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) acc += a[k] * r[k];
+    }
+  } else {
+    for (int c = lane; c < W; c += 64) acc += ldf<T>(hr + c) * rr[c];
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) z[t * E + e] = acc;
+}
+
+// One wave per token: softmax over the experts' scores, then the `top` largest (lowest index on a tie),
+// divided by their sum (+ 1e-20) and multiplied by scale.
+__global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ z, int E, int top, float scale,
+                                                      int* __restrict__ idx, float* __restrict__ wts) {
   extern __shared__ __attribute__((aligned(16))) float z_s[];   // [E]
   const size_t t = blockIdx.x;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int e = wave; e < E; e += NT / 64) {
-    float acc = 0.f;
-    for (int c = lane; c < W; c += 64) acc += ldf<T>(h + t * W + c) * router[(size_t)e * W + c];
-    acc = wave_sum(acc);
-    if (lane == 0) z_s[e] = acc;
-  }
-  __syncthreads();
-  if (wave != 0) return;
+  const int lane = threadIdx.x;
   float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z_s[e]);
+  for (int e = lane; e < E; e += 64) { z_s[e] = z[t * E + e]; mx = fmaxf(mx, z_s[e]); }
   mx = wave_max(mx);
   float sum = 0.f;
   for (int e = lane; e < E; e += 64) sum += expf(z_s[e] - mx);
@@ -357,6 +405,10 @@ __global__ void __launch_bounds__(NT) moe_route_kernel(const T* __restrict__ h, 
       const int oi = __shfl_xor(bi, o, 64);
       if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
     }
+    if (bi >= E) {                                           // scores that compare with nothing (NaN): keep the ids in range
+      bi = k;
+      best = 0.f;
+    }
     if (lane == k) { my_w = best; my_i = bi; }
     if (lane == 0) z_s[bi] = -2.f;                           // LDS accesses of one wave keep their order
     tot += best;
@@ -372,13 +424,13 @@ __global__ void __launch_bounds__(NT) moe_route_kernel(const T* __restrict__ h, 
 template <typename T>
 __global__ void __launch_bounds__(NT) moe_gate_up_kernel(const T* __restrict__ h, int W, const int* __restrict__ idx, int top,
                                                          const T* __restrict__ w_gu, int ff, float limit, T* __restrict__ y,
-                                                         int rows_per_wg) {
+                                                         int rows_per_wg, int E) {
   extern __shared__ __attribute__((aligned(16))) float h_s[];   // [W]
   const size_t pair = blockIdx.x, t = pair / top;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int c = tid; c < W; c += NT) h_s[c] = ldf<T>(h + t * W + c);
   __syncthreads();
-  const T* wg = w_gu + (size_t)idx[pair] * 2 * ff * W;
+  const T* wg = w_gu + (size_t)min(max(idx[pair], 0), E - 1) * 2 * ff * W;
   const int r1 = min(ff, (int)(blockIdx.y + 1) * rows_per_wg);
   for (int r = blockIdx.y * rows_per_wg + wave; r < r1; r += NT / 64) {
     float ag = 0.f, au = 0.f;
@@ -405,13 +457,13 @@ __global__ void __launch_bounds__(NT) moe_gate_up_kernel(const T* __restrict__ h
 template <typename T>
 __global__ void __launch_bounds__(NT) moe_down_kernel(const T* __restrict__ y, int ff, const int* __restrict__ idx,
                                                       const T* __restrict__ w_down, int W, T* __restrict__ out,
-                                                      int rows_per_wg) {
+                                                      int rows_per_wg, int E) {
   extern __shared__ __attribute__((aligned(16))) float y_s[];   // [ff]
   const size_t pair = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int c = tid; c < ff; c += NT) y_s[c] = ldf<T>(y + pair * ff + c);
   __syncthreads();
-  const T* wd = w_down + (size_t)idx[pair] * W * ff;
+  const T* wd = w_down + (size_t)min(max(idx[pair], 0), E - 1) * W * ff;
   const int r1 = min(W, (int)(blockIdx.y + 1) * rows_per_wg);
   for (int r = blockIdx.y * rows_per_wg + wave; r < r1; r += NT / 64) {
     float acc = 0.f;
@@ -531,37 +583,38 @@ int edge_sm_delta_scan(const float* prep, int prep_ld, const void* qkv, int Cq, 
                        int P, int f32, hipStream_t st) {
   if (n == 0) return 0;
   if (G <= 0 || H % G || N > 256) return -2;
-  const dim3 grid(n, H, (P + 63) / 64);
+  const dim3 grid(n, H, (P + 15) / 16);
 #define SM_DS(NR)                                                                                                  \
   SM_T(f32, hipLaunchKernelGGL((delta_scan_kernel<T, NR>), grid, dim3(NT), 0, st, prep, prep_ld, (const T*)qkv, Cq, \
                                state, seq_slot, seq_start, seq_len, seq_off, y, H, G, N, P))
-  if (N <= 32) SM_DS(8);
-  else if (N <= 64) SM_DS(16);
-  else if (N <= 128) SM_DS(32);
-  else SM_DS(64);
+  if (N <= 64) SM_DS(4);
+  else if (N <= 128) SM_DS(8);
+  else SM_DS(16);
 #undef SM_DS
   return (int)hipGetLastError();
 }
 
-int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, int* idx, float* wts, int rows,
-                      int f32, hipStream_t st) {
+// z: fp32 scratch [rows, E] (the experts' scores)
+int edge_sm_moe_route(const void* h, int W, const float* router, int E, int top, float scale, float* z, int* idx, float* wts,
+                      int rows, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   if (top < 1 || top > E || top > 64 || E > 8192) return -2;
-  SM_T(f32, hipLaunchKernelGGL(moe_route_kernel<T>, dim3(rows), dim3(NT), (size_t)E * 4, st, (const T*)h, W, router, E, top,
-                               scale, idx, wts));
+  SM_T(f32, hipLaunchKernelGGL(moe_logits_kernel<T>, dim3(rows, (E + NT / 64 - 1) / (NT / 64)), dim3(NT), 0, st, (const T*)h,
+                               W, router, E, z));
+  hipLaunchKernelGGL(moe_topk_kernel, dim3(rows), dim3(64), (size_t)E * 4, st, (const float*)z, E, top, scale, idx, wts);
   return (int)hipGetLastError();
 }
 
 // y: scratch [rows * top, ff]; out [rows * top, W]
 int edge_sm_moe_experts(const void* h, int W, const int* idx, int top, const void* w_gu, const void* w_down, int ff,
-                        float limit, void* y, void* out, int rows, int f32, hipStream_t st) {
+                        float limit, void* y, void* out, int rows, int E, int f32, hipStream_t st) {
   if (rows == 0) return 0;
   if ((size_t)W * 4 > 60 * 1024 || (size_t)ff * 4 > 60 * 1024) return -3;
   const int rpw = 16;
   SM_T(f32, hipLaunchKernelGGL(moe_gate_up_kernel<T>, dim3(rows * top, (ff + rpw - 1) / rpw), dim3(NT), (size_t)W * 4, st,
-                               (const T*)h, W, idx, top, (const T*)w_gu, ff, limit, (T*)y, rpw));
+                               (const T*)h, W, idx, top, (const T*)w_gu, ff, limit, (T*)y, rpw, E));
   SM_T(f32, hipLaunchKernelGGL(moe_down_kernel<T>, dim3(rows * top, (W + rpw - 1) / rpw), dim3(NT), (size_t)ff * 4, st,
-                               (const T*)y, ff, idx, (const T*)w_down, W, (T*)out, rpw));
+                               (const T*)y, ff, idx, (const T*)w_down, W, (T*)out, rpw, E));
   return (int)hipGetLastError();
 }
 

@@ -462,7 +462,9 @@ constexpr int MQ = 64, MK = 64;
 // RH query heads of one kv head per workgroup: a staged key / value tile serves all of them
 // (second launch bound: workgroups per CU the register budget must allow - four for 64-wide heads, so the
 // 1024 workgroups of a 4096-token, 16-head prompt are resident at once)
-template <int DK, int DV, int RH>
+// KVS: the value of a cached row is its first Dv numbers (a latent cache): the staged key tile serves as
+// the value tile, nothing is loaded twice
+template <int DK, int DV, int RH, bool KVS>
 __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1))) attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ gate, int gate_ld, const bf16_t* __restrict__ kp,
     const bf16_t* __restrict__ vp, const float* __restrict__ kb, const float* __restrict__ vb,
@@ -470,9 +472,11 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
     const int* __restrict__ seq_off, const int* __restrict__ ptab, int ptab_ld, bf16_t* __restrict__ out, int n, int H,
     int G, int PB, float scale_log2, int window, int pool, int kld, int vld) {
   constexpr int D = 32 * DK, Dv = 16 * DV;
-  constexpr int KS = D * 2 + 16, VS = Dv * 2 + 16, PS = MK * 2 + 16;      // LDS row strides in bytes
+  constexpr int KS = D * 2 + 16, VS = KVS ? KS : Dv * 2 + 16, PS = MK * 2 + 16;      // LDS row strides in bytes
+  static_assert(!KVS || Dv <= D, "a value slice lies inside the key row");
   __shared__ __attribute__((aligned(16))) char k_lds[MK * KS];
-  __shared__ __attribute__((aligned(16))) char v_lds[MK * VS];
+  __shared__ __attribute__((aligned(16))) char v_own[KVS ? 16 : MK * VS];
+  char* const v_lds = KVS ? k_lds : v_own;
   __shared__ __attribute__((aligned(16))) char p_all[4 * 16 * PS];
   constexpr int NPID = 1024;
   __shared__ int pid_s[NPID];                                // the sequence's first page ids (one global hop per tile less)
@@ -520,8 +524,8 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
   // a tile's rows travel global -> registers while the tile before it computes, registers -> LDS
   // between the two barriers
   static_assert(DV % 2 == 0, "value chunks per thread");
-  constexpr int KL = DK, VL = DV / 2;                        // 16-byte chunks per thread per tile
-  uint4 kreg[KL], vreg[VL];
+  constexpr int KL = DK, VL = KVS ? 0 : DV / 2;              // 16-byte chunks per thread per tile
+  uint4 kreg[KL], vreg[VL > 0 ? VL : 1];
   auto load_tile = [&](int tile) {
     const bool tok = tile < tok_tiles;
     const int base = tok ? (jlo / MK + tile) * MK : (tile - tok_tiles) * MK;
@@ -543,7 +547,7 @@ __global__ void __launch_bounds__(NT, (DV * RH <= 4 ? 4 : (DV * RH <= 8 ? 2 : 1)
         v = pack8(f);
       }
       if (isk) kreg[i] = v;
-      else vreg[i - KL] = v;
+      else vreg[VL > 0 ? i - KL : 0] = v;
     }
   };
   auto store_tile = [&]() {
@@ -1262,28 +1266,43 @@ int edge_sm_attention_mfma(const void* q, const void* gate, int gate_ld, const v
   int rh = 1;
   if (R % 4 == 0 && (long)qtiles * (H / 4) >= 1024) rh = 4;
   else if (R % 2 == 0 && (long)qtiles * (H / 2) >= 1024) rh = 2;
-#define SM_MF_R(DK, DV, RH)                                                                                        \
-  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV, RH>), dim3(qtiles, H / RH), dim3(NT), 0, st, (const bf16_t*)q,     \
-                     (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb, seq_slot,         \
-                     seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window, pool, kld, vld)
-#define SM_MF(DK, DV)                      \
-  do {                                     \
-    if (rh == 4) SM_MF_R(DK, DV, 4);       \
-    else if (rh == 2) SM_MF_R(DK, DV, 2);  \
-    else SM_MF_R(DK, DV, 1);               \
+  const bool kvs = kp == vp && kld == vld;
+  if (kvs && pool > 0) return 1;                             // pooled entries keep separate key / value rows
+#define SM_MF_ARGS                                                                                                  \
+  dim3(NT), 0, st, (const bf16_t*)q, (const bf16_t*)gate, gate_ld, (const bf16_t*)kp, (const bf16_t*)vp, kb, vb,     \
+      seq_slot, seq_start, seq_len, seq_off, ptab, ptab_ld, (bf16_t*)out, n, H, G, PB, sl2, window, pool, kld, vld
+#define SM_MF_R(DK, DV, RH, KVS) \
+  hipLaunchKernelGGL((attn_mfma_kernel<DK, DV, RH, KVS>), dim3(qtiles, H / RH), SM_MF_ARGS)
+#define SM_MF(DK, DV)                             \
+  do {                                            \
+    if (rh == 4) SM_MF_R(DK, DV, 4, false);       \
+    else if (rh == 2) SM_MF_R(DK, DV, 2, false);  \
+    else SM_MF_R(DK, DV, 1, false);               \
   } while (0)
-  if (D == 64 && Dv == 64) SM_MF(2, 4);
+#define SM_MFK(DK, DV)                            \
+  do {                                            \
+    if (rh == 4) SM_MF_R(DK, DV, 4, true);        \
+    else if (rh == 2) SM_MF_R(DK, DV, 2, true);   \
+    else SM_MF_R(DK, DV, 1, true);                \
+  } while (0)
+  if (kvs) {                                                 // latent rows: latent | shared key part, value = the latent
+    if (D == 128 && Dv == 96) SM_MFK(4, 6);
+    else if (D == 160 && Dv == 128) SM_MFK(5, 8);
+    else if (D == 192 && Dv == 128) SM_MFK(6, 8);
+    else if (D == 320 && Dv == 256) SM_MF_R(10, 16, 1, true);   // one head per workgroup: its output tile fills the registers
+    else return 1;
+  }
+  else if (D == 64 && Dv == 64) SM_MF(2, 4);
   else if (D == 96 && Dv == 96) SM_MF(3, 6);
   else if (D == 128 && Dv == 128) SM_MF(4, 8);
   else if (D == 128 && Dv == 64) SM_MF(4, 4);
   else if (D == 64 && Dv == 128) SM_MF(2, 8);
   else if (D == 32 && Dv == 32) SM_MF(1, 2);
-  else if (D == 128 && Dv == 96) SM_MF(4, 6);                // latent rows: latent + shared key part, value = the latent
-  else if (D == 160 && Dv == 128) SM_MF(5, 8);
-  else if (D == 192 && Dv == 128) SM_MF(6, 8);
   else return 1;
 #undef SM_MF
+#undef SM_MFK
 #undef SM_MF_R
+#undef SM_MF_ARGS
   return (int)hipGetLastError();
 }
 

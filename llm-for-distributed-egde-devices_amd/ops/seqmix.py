@@ -572,22 +572,26 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gu: torch.Tensor, w_down: 
 
 
 def _moe_experts_sorted(h, idx, w_gu, w_down, limit):
-    """Prompt-sized steps: (token, choice) pairs sorted by expert, one pair of vendor GEMMs per expert
-    over its rows (the counts cross to the host once per call)."""
+    """Prompt-sized steps: (token, choice) pairs sorted by expert (the counts cross to the host once per
+    call); one vendor GEMM per expert over its rows for gate | up, one activation launch over all
+    rows, one vendor GEMM per expert for down, and the rows go back to (token, choice) order."""
     T, top = idx.shape
     E, ff2, W = w_gu.shape
-    flat = idx.reshape(-1).long()
+    flat = idx.reshape(-1).long().clamp_(0, E - 1)
     order = torch.argsort(flat, stable=True)
     counts = torch.bincount(flat, minlength=E).tolist()
     rows = h.index_select(0, order // top)
-    y = torch.empty(T * top, ff2 // 2, dtype=h.dtype, device=h.device)
+    u = torch.empty(T * top, ff2, dtype=h.dtype, device=h.device)
     o = torch.empty(T * top, w_down.shape[1], dtype=h.dtype, device=h.device)
-    a = 0
+    spans, a = [], 0
     for e, n in enumerate(counts):
         if n:
-            y[a:a + n] = glu_clamp(F.linear(rows[a:a + n], w_gu[e]), ff2 // 2, limit)
-            torch.mm(y[a:a + n], w_down[e].t(), out=o[a:a + n])
+            spans.append((e, a, n))
+            torch.mm(rows[a:a + n], w_gu[e].t(), out=u[a:a + n])
             a += n
-    out = torch.empty_like(o)
-    out[order] = o
-    return out.view(T, top, -1)
+    y = glu_clamp(u, ff2 // 2, limit)
+    for e, a, n in spans:
+        torch.mm(y[a:a + n], w_down[e].t(), out=o[a:a + n])
+    back = torch.empty_like(order)
+    back[order] = torch.arange(T * top, device=h.device)
+    return o.index_select(0, back).view(T, top, -1)

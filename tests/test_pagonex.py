@@ -360,6 +360,16 @@ def test_router_and_experts(dev, T):
     got = (wts[..., None] * parts.float()).sum(1).cpu().double()
     assert torch.allclose(got, want, atol=2e-5, rtol=1e-4)
     assert torch.allclose(wts.sum(-1).cpu(), torch.full((T,), 2.0), atol=1e-5)
+    # a skewed routing (nearly every token to the same experts) takes the per-expert path of prompt-sized steps
+    skew = torch.zeros(T, top, dtype=torch.int32)
+    skew[:, 1], skew[:, 2] = 1, 2
+    skew[0] = torch.tensor([5, 4, 3])
+    one = seqmix.moe_experts(D(h), D(skew), D(w_gu), D(w_down), 1.0).cpu().double()
+    for t in (0, 1, T - 1):
+        for k in range(top):
+            e = int(skew[t, k])
+            assert torch.allclose(one[t, k], oracle.expert(h[t:t + 1].double(), {n: v.double() for n, v in w.items()}, f"e{e}.", 1.0)[0],
+                                  atol=2e-5, rtol=1e-4)
 
 
 # --------------------------------------------------------------------------- whole models
@@ -575,7 +585,7 @@ def test_decode_graph_replays_match_eager(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kv_rank,rot_dim,heads", [(96, 32, 6), (128, 64, 16), (24, 8, 3)])
+@pytest.mark.parametrize("kv_rank,rot_dim,heads", [(96, 32, 6), (128, 64, 16), (24, 8, 3), (128, 32, 4), (256, 64, 8), (512, 64, 2)])
 def test_bf16_prompt_attention_over_latent_rows(kv_rank, rot_dim, heads):
     """The attention op on bf16 latent rows (value = the first kv_rank numbers of the key row) for prompt
     portions (the matrix-core kernel where it takes the sizes) against the same op in fp32 on the CPU."""
