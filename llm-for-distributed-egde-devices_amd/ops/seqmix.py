@@ -572,26 +572,33 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, w_gu: torch.Tensor, w_down: 
 
 
 def _moe_experts_sorted(h, idx, w_gu, w_down, limit):
-    """Prompt-sized steps: (token, choice) pairs sorted by expert (the counts cross to the host once per
-    call); one vendor GEMM per expert over its rows for gate | up, one activation launch over all
-    rows, one vendor GEMM per expert for down, and the rows go back to (token, choice) order."""
+    """Prompt-sized steps: (token, choice) pairs sorted by expert; every expert's rows run through its
+    gate | up weights, one activation launch covers all rows, every expert's rows run through its down
+    weights, and the rows go back to (token, choice) order.  bf16 on the GPU: the library's grouped
+    product over the sorted rows with the experts' end offsets on the device (nothing crosses to the
+    host, so the step stays asynchronous); otherwise one GEMM per expert with the counts on the host."""
     T, top = idx.shape
     E, ff2, W = w_gu.shape
     flat = idx.reshape(-1).long().clamp_(0, E - 1)
     order = torch.argsort(flat, stable=True)
-    counts = torch.bincount(flat, minlength=E).tolist()
+    counts = torch.bincount(flat, minlength=E)
     rows = h.index_select(0, order // top)
-    u = torch.empty(T * top, ff2, dtype=h.dtype, device=h.device)
-    o = torch.empty(T * top, w_down.shape[1], dtype=h.dtype, device=h.device)
-    spans, a = [], 0
-    for e, n in enumerate(counts):
-        if n:
-            spans.append((e, a, n))
-            torch.mm(rows[a:a + n], w_gu[e].t(), out=u[a:a + n])
-            a += n
-    y = glu_clamp(u, ff2 // 2, limit)
-    for e, a, n in spans:
-        torch.mm(y[a:a + n], w_down[e].t(), out=o[a:a + n])
+    if h.is_cuda and h.dtype == torch.bfloat16 and W % 8 == 0 and ff2 % 16 == 0 and hasattr(torch, "_grouped_mm"):
+        ends = torch.cumsum(counts, 0).to(torch.int32)
+        y = glu_clamp(torch._grouped_mm(rows, w_gu.transpose(1, 2), offs=ends), ff2 // 2, limit)
+        o = torch._grouped_mm(y, w_down.transpose(1, 2), offs=ends)
+    else:
+        u = torch.empty(T * top, ff2, dtype=h.dtype, device=h.device)
+        o = torch.empty(T * top, w_down.shape[1], dtype=h.dtype, device=h.device)
+        spans, a = [], 0
+        for e, n in enumerate(counts.tolist()):
+            if n:
+                spans.append((e, a, n))
+                torch.mm(rows[a:a + n], w_gu[e].t(), out=u[a:a + n])
+                a += n
+        y = glu_clamp(u, ff2 // 2, limit)
+        for e, a, n in spans:
+            torch.mm(y[a:a + n], w_down[e].t(), out=o[a:a + n])
     back = torch.empty_like(order)
     back[order] = torch.arange(T * top, device=h.device)
     return o.index_select(0, back).view(T, top, -1)

@@ -585,6 +585,23 @@ def test_decode_graph_replays_match_eager(tmp_path):
 
 
 @pytest.mark.gpu
+def test_bf16_prompt_sized_experts_against_the_decode_sized_path():
+    """The sorted path of prompt-sized steps (bf16: the library's grouped product; an expert that no token
+    chose among them) against the per-pair kernels of decode-sized steps."""
+    torch.manual_seed(4)
+    T, W, E, top, ff = 150, 64, 7, 2, 48
+    h = torch.randn(T, W, device="cuda").bfloat16()
+    w_gu = (torch.randn(E, 2 * ff, W, device="cuda") * 0.2).bfloat16()
+    w_down = (torch.randn(E, W, ff, device="cuda") * 0.2).bfloat16()
+    idx = torch.randint(0, E - 1, (T, top), device="cuda", dtype=torch.int32)      # expert E - 1 stays idle
+    idx[:, 1] = (idx[:, 0] + 1) % (E - 1)
+    big = seqmix.moe_experts(h, idx, w_gu, w_down, 1.5).float()
+    small = torch.cat([seqmix.moe_experts(h[a:a + 50].contiguous(), idx[a:a + 50].contiguous(), w_gu, w_down, 1.5)
+                       for a in range(0, T, 50)]).float()
+    assert torch.allclose(big, small, atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("kv_rank,rot_dim,heads", [(96, 32, 6), (128, 64, 16), (24, 8, 3), (128, 32, 4), (256, 64, 8), (512, 64, 2)])
 def test_bf16_prompt_attention_over_latent_rows(kv_rank, rot_dim, heads):
     """The attention op on bf16 latent rows (value = the first kv_rank numbers of the key row) for prompt
