@@ -47,7 +47,8 @@ __global__ void prev_token_kernel(const int64_t* __restrict__ ids, int64_t* __re
 // out = x + sum_k w[:, k] x_(pos - taps + 1 + k) over the fp32 stream; inputs before the portion come from
 // the slot's tail (zeros before the sequence's start).  state_w: steps in which every sequence brings one
 // token shift the tail in the same launch (the thread of (token, channel) is that channel's only reader).
-template <typename T>
+// VEC: four channels per thread through 16-byte loads of the stream (W a multiple of 4)
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(NT) canon_kernel(const float* __restrict__ x, int W, const float* __restrict__ w,
                                                    const float* state, const int* __restrict__ tok_seq,
                                                    const int* __restrict__ tok_pos, const int* __restrict__ seq_slot,
@@ -56,6 +57,28 @@ __global__ void __launch_bounds__(NT) canon_kernel(const float* __restrict__ x, 
   const int t = blockIdx.x, s = tok_seq[t], pos = tok_pos[t], start = seq_start[s], off = seq_off[s];
   const float* st = state + (size_t)seq_slot[s] * (taps - 1) * W;
   float* stw = state_w ? state_w + (size_t)seq_slot[s] * (taps - 1) * W : nullptr;
+  if constexpr (VEC) {
+    for (int c = (blockIdx.y * NT + threadIdx.x) * 4; c < W; c += NT * gridDim.y * 4) {
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int k = 0; k < taps; ++k) {
+        const int p = pos - (taps - 1) + k;
+        v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (p >= start) v = *reinterpret_cast<const float4*>(x + (size_t)(off + p - start) * W + c);
+        else if (p >= 0) v = *reinterpret_cast<const float4*>(st + (size_t)(p - (start - (taps - 1))) * W + c);
+        acc[0] += w[c * taps + k] * v.x;
+        acc[1] += w[(c + 1) * taps + k] * v.y;
+        acc[2] += w[(c + 2) * taps + k] * v.z;
+        acc[3] += w[(c + 3) * taps + k] * v.w;
+        if (stw && k >= 1) *reinterpret_cast<float4*>(stw + (size_t)(k - 1) * W + c) = v;
+      }
+      stf<T>(out + (size_t)t * W + c, v.x + acc[0]);
+      stf<T>(out + (size_t)t * W + c + 1, v.y + acc[1]);
+      stf<T>(out + (size_t)t * W + c + 2, v.z + acc[2]);
+      stf<T>(out + (size_t)t * W + c + 3, v.w + acc[3]);
+    }
+    return;
+  }
   for (int c = blockIdx.y * NT + threadIdx.x; c < W; c += NT * gridDim.y) {
     float acc = 0.f, cur = 0.f;
     for (int k = 0; k < taps; ++k) {
@@ -511,8 +534,14 @@ int edge_sm_canon(const float* x, int W, const float* w, float* state, const int
   if (taps < 1 || taps > 16) return -2;
   const bool one = max_len == 1 && taps > 1;                 // every sequence brings one token
   const int gy = (W + NT * 4 - 1) / (NT * 4);
-  SM_T(f32, hipLaunchKernelGGL(canon_kernel<T>, dim3(rows, gy), dim3(NT), 0, st, x, W, w, (const float*)state, tok_seq,
-                               tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps, one ? state : (float*)nullptr));
+  if (W % 4 == 0)
+    SM_T(f32, hipLaunchKernelGGL((canon_kernel<T, true>), dim3(rows, gy), dim3(NT), 0, st, x, W, w, (const float*)state,
+                                 tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps,
+                                 one ? state : (float*)nullptr));
+  else
+    SM_T(f32, hipLaunchKernelGGL((canon_kernel<T, false>), dim3(rows, gy), dim3(NT), 0, st, x, W, w, (const float*)state,
+                                 tok_seq, tok_pos, seq_slot, seq_start, seq_off, (T*)out, taps,
+                                 one ? state : (float*)nullptr));
   if (taps > 1 && !one)
     hipLaunchKernelGGL(canon_state_kernel, dim3(n, gy), dim3(NT), 0, st, x, W, state, seq_slot, seq_start, seq_len, seq_off,
                        taps);

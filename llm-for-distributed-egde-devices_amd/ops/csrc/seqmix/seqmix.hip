@@ -1130,16 +1130,19 @@ static size_t attn_lds_bytes(int rmax, int D, int Dv) {
 }
 
 // query heads of one kv head that share a workgroup: the whole group up to 16, fewer while their rows
-// (queries, scores, partial outputs) would not fit 64 KB of LDS; 0: not even one head fits
-int edge_sm_attention_rmax(int H, int G, int D, int Dv) {
+// (queries, scores, partial outputs) would not fit 64 KB of LDS, and down to 4 while a step of few
+// queries over few kv heads (decode steps over one latent head) would leave most CUs without a
+// workgroup; 0: not even one head fits
+int edge_sm_attention_rmax(int rows, int H, int G, int D, int Dv) {
   const int R = H / G;
   int rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16;
   while (rmax > 1 && attn_lds_bytes(rmax, D, Dv) > 64 * 1024) rmax >>= 1;
+  while (rmax > 4 && (long)rows * G * ((R + rmax - 1) / rmax) < 64) rmax >>= 1;
   return attn_lds_bytes(rmax, D, Dv) > 64 * 1024 ? 0 : rmax;
 }
 
 size_t edge_sm_attention_part_floats(int rows, int H, int G, int D, int Dv, int nsplit) {
-  const int R = H / G, rmax = max(1, edge_sm_attention_rmax(H, G, D, Dv)), nsp = (R + rmax - 1) / rmax;
+  const int R = H / G, rmax = max(1, edge_sm_attention_rmax(rows, H, G, D, Dv)), nsp = (R + rmax - 1) / rmax;
   return (size_t)rows * G * nsp * nsplit * rmax * (Dv + 2);
 }
 
@@ -1150,7 +1153,7 @@ int edge_sm_attention(const void* q, const void* gate, int gate_ld, const void* 
   if (rows == 0) return 0;
   if (G <= 0 || H % G || Dv > 512) return -2;
   const int R = H / G;
-  const int rmax = edge_sm_attention_rmax(H, G, D, Dv);
+  const int rmax = edge_sm_attention_rmax(rows, H, G, D, Dv);
   if (rmax == 0) return -3;
   const int nsp = (R + rmax - 1) / rmax;
   if (nsplit < 1 || (nsplit > 1 && !part)) return -2;
