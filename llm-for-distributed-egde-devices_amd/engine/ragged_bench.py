@@ -63,7 +63,7 @@ PAGONEX_SIZES = {
 
 def pagonex_config(s: dict) -> ModelConfig:
     yarn = {"rope_type": "yarn", "factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
-    moe = MoESpec(s["experts"], s["top"], 2.5, s["ff"], 7.0, s["shared"], 7.0)
+    moe = MoESpec(s["experts"], s["top"], 2.0, s["ff"], 7.0, s["shared"], 7.0)
     specs = []
     for i in range(s["layers"]):
         if i % 2 == 0:
@@ -78,8 +78,8 @@ def pagonex_config(s: dict) -> ModelConfig:
     return ModelConfig(arch="pagonex", vocab_size=s["vocab"], hidden_size=s["width"], num_layers=s["layers"],
                        num_heads=s["heads"], num_kv_heads=1, intermediate_size=0, head_dim=1,
                        max_position_embeddings=1 << 20, norm="layer", norm_eps=1e-6, act="glu_clamp", name="pagonex-bench",
-                       layer_specs=specs, canon_taps=3, bigram={"buckets": 8191, "mul_prev": 31, "mul_cur": 7},
-                       logit_scale=0.5)
+                       layer_specs=specs, canon_taps=4, bigram={"buckets": 8191, "mul_prev": 131, "mul_cur": 17},
+                       logit_scale=1.0)
 
 
 def closest_config(s: dict) -> ModelConfig:

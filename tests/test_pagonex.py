@@ -602,7 +602,7 @@ def test_bf16_prompt_sized_experts_against_the_decode_sized_path():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kv_rank,rot_dim,heads", [(96, 32, 6), (128, 64, 16), (24, 8, 3), (128, 32, 4), (256, 64, 8), (512, 64, 2)])
+@pytest.mark.parametrize("kv_rank,rot_dim,heads", [(96, 32, 4), (128, 64, 16), (24, 8, 3), (128, 32, 4), (256, 64, 8), (512, 64, 2)])
 def test_bf16_prompt_attention_over_latent_rows(kv_rank, rot_dim, heads):
     """The attention op on bf16 latent rows (value = the first kv_rank numbers of the key row) for prompt
     portions (the matrix-core kernel where it takes the sizes) against the same op in fp32 on the CPU."""
