@@ -1,7 +1,7 @@
 """Register-spill guard for the kernels that count their own LDS-DMA with inline
 ``s_waitcnt vmcnt(N)``: a spill's scratch loads / stores join the same counter, so a spilling
-ring kernel waits for the wrong operations and reads LDS before its DMA landed (round 2: a 10-wave
-decode kernel spilled 236 B/lane and produced non-deterministic slices).  Cross-compiles for
+ring kernel waits for the wrong operations and reads LDS before its DMA landed (a 10-wave decode
+kernel that spilled 236 B/lane produced non-deterministic slices).  Cross-compiles for
 gfx950 on the CPU (tools/kernel_resources.py) and requires zero scratch in every kernel of the
 files that hold such rings."""
 import os

@@ -585,6 +585,26 @@ def test_decode_graph_replays_match_eager(tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("width,heads,dim,rot,vdim,kvr,qr,dh,dn,dp,ff,E", [(34, 3, 5, 2, 7, 9, 11, 3, 7, 5, 9, 3), (66, 5, 6, 6, 3, 13, 7, 5, 9, 11, 13, 1),
+                                                                          (96, 12, 16, 16, 8, 48, 40, 6, 32, 24, 40, 9)])
+def test_bf16_odd_sizes(tmp_path, width, heads, dim, rot, vdim, kvr, qr, dh, dn, dp, ff, E):
+    """16-bit storage with sizes that are not multiples of 8 (unaligned slices of the fused projections,
+    scalar paths of the kernels) and one with aligned sizes, prompt-sized and decode-sized steps: the bulk of
+    the rows within 16-bit rounding of the oracle."""
+    cfg = make_config(layers=[latent(heads=heads, dim=dim, rot_dim=rot, vdim=vdim, q_rank=qr, kv_rank=kvr, window=40),
+                              delta(heads=dh, kv_heads=dh, dim=dn, vdim=dp, conv=3),
+                              latent(heads=heads, dim=dim, rot_dim=rot, vdim=vdim, q_rank=qr, kv_rank=kvr, window=70, kv_from=0)],
+                      mlps=[moe(experts=E, top=min(2, E), ff=ff, shared=ff + 1)] * 3, width=width, vocab=97)
+    w = make_weights(cfg, seed=width, decay_rank=5, gate_rank=3)
+    model = load(tmp_path, cfg, w, "cuda", precision="bf16")
+    toks = tokens(150, cfg["vocab"], 3)
+    want = oracle.forward(cfg, w, toks)
+    got, _ = replay(model, [[("a", 100)], [("a", 30)]] + [[("a", 1)]] * 20, {"a": toks}, 192)
+    e = row_err(got["a"], want)
+    assert torch.isfinite(got["a"]).all() and e.median() < 5e-2 and e.quantile(0.9) < 0.3, (e.median(), e.quantile(0.9))
+
+
+@pytest.mark.gpu
 def test_bf16_prompt_sized_experts_against_the_decode_sized_path():
     """The sorted path of prompt-sized steps (bf16: the library's grouped product; an expert that no token
     chose among them) against the per-pair kernels of decode-sized steps."""
