@@ -1807,7 +1807,7 @@ int launch_norm(const NormIn& na, const void* Wp, const float* sw, const void* b
 //    beside the partner's MFMAs), 2 weight + 2 activation loader waves, >= 4 stages per slice
 //    (down, K = 11008: 22.4 -> 20.1 us against the earlier one-ring kernel);
 //  * qkv-like EPI_OUT (3 tiles) and the quantising GLU (8 tiles = one 64-feature group) with
-//    dedicated weight loaders (the 2-lane bench 32.0k against 28.3k tok/s in round 2).
+//    dedicated weight loaders (the 2-lane bench 32.0k against 28.3k tok/s before them).
 // K % 128 == 0 (split-K: >= 4 stages per slice; rows128_ok).  The quantising GLU takes it from 33
 // rows (gate_up at 64 rows: 26.6 us here against 33.9 for the weight-stationary GEMV; the ring's
 // surplus rows are clamped reads, never stored).  -1: no kernel for this call.
