@@ -565,6 +565,66 @@ def test_checkpoint_round_trip(tmp_path):
     assert torch.allclose(a, b, atol=1e-6)
 
 
+def test_evaluate_cli_runs_a_pagonex_checkpoint(tmp_path):
+    """The evaluation command line on a checkpoint folder of this design (vocabulary wide enough for the
+    byte tokenizer): loader by config.json, paged engine and scheduler, the sampling configuration, the
+    confidence metric through the model's own prompt pass."""
+    from safetensors.torch import save_file
+    from edgellm.cli import evaluate
+    cfg = make_config(vocab=300, width=24)
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file(make_weights(cfg, seed=3), str(d / "model.safetensors"))
+    y = tmp_path / "c.yaml"
+    y.write_text(f"""
+max_new_tokens: 4
+temperature: 0.7
+top_k: 50
+top_p: 0.9
+repetition_penalty: 1.1
+dataset_name: sentence-transformers/natural-questions
+dataset_split: train[:2]
+embedder_model: "none"
+models: ["{d}"]
+""")
+    out = evaluate.main(["--config", str(y), "--devices", "cpu", "--num_samples", "2", "--max_seq", "256",
+                         "--batch_size", "2", "--prefill_chunk", "16", "--precision", "fp32"])
+    assert out[str(d)]["tps"] > 0 and 0 < out[str(d)]["confidence"] <= 1
+
+
+def test_trace_runner_program_on_a_pagonex_checkpoint(tmp_path):
+    """``bin/trace_run`` as a program: steps on standard input, logits files and ``done`` lines out; a
+    request cut into portions gives the logits of the same request in one step."""
+    import subprocess
+    import numpy as np
+    from safetensors.torch import save_file
+    cfg = make_config()
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    save_file(make_weights(cfg, seed=5), str(d / "model.safetensors"))
+    toks = tokens(20, cfg["vocab"], 6)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks, "want": [3, 19]}], "end": ["a"]},
+             {"step": 1, "entries": [{"id": "b", "tokens": toks[:7], "want": [3]}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": toks[7:19], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "b", "tokens": toks[19:], "want": [0]}], "end": ["b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(d), "--dtype", "float32", "--out",
+                        str(tmp_path / "out"), "--max-tokens", "64", "--device", "cpu"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(4)]
+    V = cfg["vocab"]
+    whole = np.fromfile(tmp_path / "out" / "0.f32", dtype="<f4").reshape(2, V)
+    first = np.fromfile(tmp_path / "out" / "1.f32", dtype="<f4").reshape(1, V)
+    last = np.fromfile(tmp_path / "out" / "3.f32", dtype="<f4").reshape(1, V)
+    assert not (tmp_path / "out" / "2.f32").exists()
+    assert np.allclose(whole[0], first[0], atol=1e-4) and np.allclose(whole[1], last[0], atol=1e-4)
+    want = oracle.forward(cfg, make_weights(cfg, seed=5), toks)
+    assert close(torch.from_numpy(whole.copy()), want[[3, 19]], TOL["fp32"])
+
+
 # --------------------------------------------------------------------------- GPU only
 @pytest.mark.gpu
 def test_decode_graph_replays_match_eager(tmp_path):
