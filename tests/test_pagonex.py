@@ -271,7 +271,7 @@ def test_norms_activation_and_expert_sum(dev):
 
 
 @pytest.mark.parametrize("dev", DEVS)
-@pytest.mark.parametrize("H,G,N,P", [(4, 2, 6, 5), (2, 2, 40, 70), (3, 1, 64, 16), (1, 1, 130, 3)])
+@pytest.mark.parametrize("H,G,N,P", [(4, 2, 6, 5), (2, 2, 40, 70), (3, 1, 64, 16), (1, 1, 130, 3), (2, 1, 100, 20)])
 def test_delta_rule_in_portions_over_stale_state(dev, H, G, N, P):
     """The recurrence alone: two interleaved sequences fed in portions of 1..7 tokens into slots whose
     state an earlier request left behind; decays well below one, so a lost or stale state shows."""
@@ -645,6 +645,59 @@ def test_decode_graph_replays_match_eager(tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("N,P", [(64, 64), (128, 48), (256, 16), (33, 130)])
+def test_delta_rule_long_portions_kernel_against_the_token_loop(N, P):
+    """Portions of 300, 65 and 1 tokens in one step, then a second step continuing each from the slots'
+    state: the kernel (many staged chunks, every register layout) against the token-by-token PyTorch form."""
+    torch.manual_seed(N)
+    H, G = 2, 1
+    res = {}
+    steps = [[300, 65, 1], [40, 200, 7]]
+    data = [(torch.randn(sum(l), 2 * G * N + H * P), torch.randn(sum(l), H), torch.randn(sum(l), H * N)) for l in steps]
+    dtb, A = torch.randn(H * N) * 0.3, torch.rand(H) - 1.5
+    for dev in ("cpu", "cuda"):
+        cache = _state_cache(dev, delta_spec=_Spec(heads=H, kv_heads=G, dim=N, vdim=P, conv=2, conv_channels=1), pages=24)
+        outs, at = [], [0, 0, 0]
+        for lens, (qkv, u, a) in zip(steps, data):
+            meta = _meta(cache, [(s, at[s], n) for s, n in enumerate(lens)], dev)
+            prep = seqmix.delta_prepare(qkv.to(dev), u.to(dev), 0, a.to(dev), dtb.to(dev), A.to(dev), H, G, N)
+            outs.append(seqmix.delta_rule_scan(prep, qkv.to(dev), cache.run(0).ssm, meta, H, G, N, P).cpu())
+            at = [x + n for x, n in zip(at, lens)]
+        res[dev] = (torch.cat(outs), cache.run(0).ssm.cpu())
+    assert torch.allclose(res["cuda"][0], res["cpu"][0], atol=2e-5, rtol=1e-4)
+    assert torch.allclose(res["cuda"][1], res["cpu"][1], atol=2e-5, rtol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kv_rank,rot_dim,heads,window", [(24, 8, 6, 600), (64, 32, 16, None), (40, 8, 5, 300), (128, 32, 3, 1000)])
+def test_decode_attention_over_long_latent_windows(kv_rank, rot_dim, heads, window, dt):
+    """One-token steps of three sequences holding 700-1100 cached latent rows: every query's keys are
+    split over several workgroups and the heads of the one kv head over several more; against the same op
+    on the CPU in fp32."""
+    torch.manual_seed(heads)
+    Dc, lens = kv_rank + rot_dim, [700, 1100, 901]
+    rows = {s: torch.randn(n, Dc).to(dt).float() for s, n in enumerate(lens)}
+    q = (torch.randn(3, heads, Dc) * 0.5).to(dt).float()
+    res = {}
+    for dev, d in (("cpu", torch.float32), ("cuda", dt)):
+        spec = _Spec(heads=heads, kv_rank=kv_rank, rot_dim=rot_dim, cache_dim=Dc, kv_from=None)
+        cache = PagedCache([_Spec(latent=spec, delta=None, moe=None, attn=None, ssd=None)], 48, slots=3, page=64, dtype=d,
+                           device=dev)
+        lat = cache.run(0).lat
+        for s, n in enumerate(lens):
+            cache.extend(s, n)
+            pos = torch.arange(n)
+            pid = cache.page_table[s, (pos // 64).to(dev)].long()
+            lat[pid, (pos % 64).to(dev), 0] = rows[s].to(dev, d)
+        meta = seqmix.RaggedMeta.build([(s, n - 1, 1) for s, n in enumerate(lens)], cache.page_table, 64, dev)
+        res[dev] = seqmix.window_pool_attention(q.to(dev, d).contiguous(), None, lat, lat[..., :kv_rank], None, None, meta,
+                                                0.2, window, None).float().cpu()
+    tol = 1e-4 if dt == torch.float32 else 2e-2
+    assert torch.allclose(res["cuda"], res["cpu"], atol=tol, rtol=tol)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("width,heads,dim,rot,vdim,kvr,qr,dh,dn,dp,ff,E", [(34, 3, 5, 2, 7, 9, 11, 3, 7, 5, 9, 3), (66, 5, 6, 6, 3, 13, 7, 5, 9, 11, 13, 1),
                                                                           (96, 12, 16, 16, 8, 48, 40, 6, 32, 24, 40, 9)])
 def test_bf16_odd_sizes(tmp_path, width, heads, dim, rot, vdim, kvr, qr, dh, dn, dp, ff, E):
@@ -682,22 +735,23 @@ def test_bf16_prompt_sized_experts_against_the_decode_sized_path():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("T,window,cuts", [(200, 70, (130, 70)), (900, 600, (500, 336, 64)), (500, None, (257, 243))])
 @pytest.mark.parametrize("kv_rank,rot_dim,heads", [(96, 32, 4), (128, 64, 16), (24, 8, 3), (128, 32, 4), (256, 64, 8), (512, 64, 2)])
-def test_bf16_prompt_attention_over_latent_rows(kv_rank, rot_dim, heads):
+def test_bf16_prompt_attention_over_latent_rows(kv_rank, rot_dim, heads, T, window, cuts):
     """The attention op on bf16 latent rows (value = the first kv_rank numbers of the key row) for prompt
     portions (the matrix-core kernel where it takes the sizes) against the same op in fp32 on the CPU."""
     torch.manual_seed(kv_rank)
-    T, window, Dc = 200, 70, kv_rank + rot_dim
+    Dc = kv_rank + rot_dim
     q = (torch.randn(T, heads, Dc) * 0.5).bfloat16().float()
     rows = torch.randn(T, Dc).bfloat16().float()
     res = {}
     for dev, dt in (("cpu", torch.float32), ("cuda", torch.bfloat16)):
         spec = _Spec(heads=heads, kv_rank=kv_rank, rot_dim=rot_dim, cache_dim=Dc, kv_from=None)
-        cache = PagedCache([_Spec(latent=spec, delta=None, moe=None, attn=None, ssd=None)], 8, slots=3, page=64, dtype=dt,
+        cache = PagedCache([_Spec(latent=spec, delta=None, moe=None, attn=None, ssd=None)], 16, slots=3, page=64, dtype=dt,
                            device=dev)
         lat = cache.run(0).lat
         out, at = [], 0
-        for n in (130, 70):
+        for n in cuts:
             meta = _meta(cache, [(1, at, n)], dev)
             pos = torch.arange(at, at + n)
             pid = cache.page_table[1, (pos // 64).to(dev)].long()
