@@ -340,12 +340,12 @@ def test_delta_rule_batch_of_sequences_in_one_call(dev):
 
 
 @pytest.mark.parametrize("dev", DEVS)
-@pytest.mark.parametrize("T", [5, 90])
-def test_router_and_experts(dev, T):
+@pytest.mark.parametrize("T,E,top", [(5, 6, 3), (90, 6, 3), (7, 70, 5), (130, 70, 5)])
+def test_router_and_experts(dev, T, E, top):
     """Router choice and weights, and the experts' outputs, for a decode-sized and a prompt-sized step
     (the two expert paths), against the per-token loop."""
     torch.manual_seed(T)
-    W, E, top, ff = 24, 6, 3, 10
+    W, ff = 24, 10
     cfgm = {"router": {"experts": E, "top": top, "scale": 2.0}, "expert": {"ff": ff, "limit": 1.0}}
     w = {"router": torch.randn(E, W)}
     for e in range(E):
@@ -361,9 +361,8 @@ def test_router_and_experts(dev, T):
     assert torch.allclose(got, want, atol=2e-5, rtol=1e-4)
     assert torch.allclose(wts.sum(-1).cpu(), torch.full((T,), 2.0), atol=1e-5)
     # a skewed routing (nearly every token to the same experts) takes the per-expert path of prompt-sized steps
-    skew = torch.zeros(T, top, dtype=torch.int32)
-    skew[:, 1], skew[:, 2] = 1, 2
-    skew[0] = torch.tensor([5, 4, 3])
+    skew = torch.arange(top, dtype=torch.int32).repeat(T, 1)
+    skew[0] = torch.arange(E - top, E, dtype=torch.int32).flip(0)
     one = seqmix.moe_experts(D(h), D(skew), D(w_gu), D(w_down), 1.0).cpu().double()
     for t in (0, 1, T - 1):
         for k in range(top):
